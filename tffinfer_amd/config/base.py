@@ -45,11 +45,13 @@ class LayerCall:
     ``layer`` indexes ``layer_specs()``.  ``cache`` names the cache (or state)
     this call works on; two calls with the same ``cache`` share it, and
     ``writes_cache=False`` makes the call a reader of a cache another call
-    fills.
+    fills.  ``offset`` >= 0: that row of the model's table of stream offsets
+    (``ModelConfig.stream_offset_rows``) is added to the stream before the call.
     """
     layer: int
     cache: int
     writes_cache: bool = True
+    offset: int = -1
 
 
 class ModelConfig:
@@ -90,6 +92,14 @@ class ModelConfig:
 
     def final_norm_spec(self) -> PartSpec:
         raise NotImplementedError
+
+    def embedding_norm_spec(self) -> PartSpec | None:
+        """A norm right after the embedding, or None."""
+        return None
+
+    def stream_offset_rows(self) -> int:
+        """Rows of the table of vectors that the run order adds to the stream (``LayerCall.offset``); 0: none."""
+        return 0
 
 
 def require(d: dict, key: str, typ, where: str = "config.json"):

@@ -1,0 +1,302 @@
+// The gated delta rule: a linear recurrence whose state, a matrix S [key channel, value channel]
+// per request and head, is decayed, corrected towards the token's value along the token's key,
+// and read with the token's query:
+//
+//   S <- g_t S;   u_t = beta_t (v_t - S^T k_t);   S <- S + k_t u_t^T;   o_t = S^T q_t
+//
+// with g_t = exp(-exp(A) softplus(a_t + dt)) and beta_t = sigmoid(b_t) per head, k_t a unit vector,
+// q_t a unit vector times dim^(-1/2).  q, k, v come from a projection through a short causal
+// convolution over time per channel and silu; the convolution's last taps - 1 inputs are part of
+// the request's state, behind the heads' matrices.  Everything here is float32.
+//
+// A request's state row: [heads][value channel][key channel] (S transposed: the key channels of one
+// value channel lie side by side, as the lanes that share the channel read them), then
+// [taps - 1][channels] of the convolution's inputs, oldest first; channels are q (kv_heads x dim),
+// k (kv_heads x dim), v (heads x vdim), in the projection's column order.
+//
+// tff_gdelta_prep:        per token: convolution + silu of q, k, v, unit vectors, beta and the decay.
+// tff_gdelta_recurrence:  the recurrence over each request's tokens of the step; also leaves the
+//                         convolution's last inputs in the state.
+// tff_head_norm_silu_gate: out = o / sqrt(mean over the head of o^2 + eps) * w[channel] * silu(gate).
+// tff_sigmoid_gate_heads: out = o * sigmoid(gate) * scale, heads of o a stride apart.
+#include "common.h"
+#include "tffinfer_kernels.h"
+
+#define GD_MAX_TAPS 8
+
+__device__ __forceinline__ float gd_silu(float z) { return z / (1.0f + expf(-z)); }
+
+// One wave per (token, unit); units: kv_heads q heads, kv_heads k heads, heads v heads, one for beta and decay.
+__global__ __launch_bounds__(64) void gdelta_prep_kernel(
+    const float* __restrict__ proj, size_t ldp, const float* __restrict__ wconv, int taps,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, const float* __restrict__ state,
+    size_t state_row, size_t tail_off, const int32_t* __restrict__ token_req, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ state_slots, float* __restrict__ pre, int H, int G, int D, int E) {
+    const int t = blockIdx.x, u = blockIdx.y, lane = threadIdx.x;
+    const int C = 2 * G * D + H * E;
+    const size_t ldq = (size_t)C + 2 * H;
+    const float* row = proj + (size_t)t * ldp;
+    float* out = pre + (size_t)t * ldq;
+    if (u == 2 * G + H) {
+        for (int h = lane; h < H; h += 64) {
+            const float b = row[C + h], a = row[C + H + h] + dt_bias[h];
+            const float sp = a > 20.f ? a : log1pf(expf(a));
+            out[C + h] = 1.0f / (1.0f + expf(-b));
+            out[C + H + h] = expf(-expf(a_log[h]) * sp);
+        }
+        return;
+    }
+    const int r = token_req[t];
+    const int i = t - cu_tokens[r];               // the token's place in its request's portion
+    const float* tail = state + (size_t)state_slots[r] * state_row + tail_off;
+    int c0, n;
+    if (u < 2 * G) { c0 = u * D; n = D; } else { c0 = 2 * G * D + (u - 2 * G) * E; n = E; }
+    float ss = 0.f;
+    for (int e = lane; e < n; e += 64) {
+        const int c = c0 + e;
+        float acc = 0.f;
+        for (int k = 0; k < taps; ++k) {
+            const int s = i - (taps - 1) + k;     // the input's place in the portion; before it: the state's
+            const float x = s >= 0 ? proj[(size_t)(t - (taps - 1) + k) * ldp + c] : tail[(size_t)(i + k) * C + c];
+            acc = fmaf(wconv[(size_t)c * taps + k], x, acc);
+        }
+        const float y = gd_silu(acc);
+        out[c] = y;
+        ss = fmaf(y, y, ss);
+    }
+    if (u < 2 * G) {
+        ss = wave_sum(ss);
+        const float f = (1.0f / sqrtf(ss + 1e-6f)) * (u < G ? 1.0f / sqrtf((float)D) : 1.0f);
+        __syncthreads();
+        for (int e = lane; e < n; e += 64) out[c0 + e] *= f;      // (each lane rescales what it wrote)
+    }
+}
+
+TFF_API int tff_gdelta_prep(const float* proj, size_t ldp, const float* wconv, int taps, const float* a_log,
+                            const float* dt_bias, const float* state, size_t state_row, size_t tail_off,
+                            const int32_t* token_req, const int32_t* cu_tokens, const int32_t* state_slots, float* pre,
+                            int T, int H, int G, int D, int E, tff_stream_t stream) {
+    TFF_REQUIRE(proj && wconv && a_log && dt_bias && state && token_req && cu_tokens && state_slots && pre,
+                "gdelta_prep: null pointer");
+    TFF_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && E > 0 && taps >= 1 && taps <= GD_MAX_TAPS,
+                "gdelta_prep: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d taps=%d (taps up to %d)", H, G, D, E, taps,
+                GD_MAX_TAPS);
+    const size_t C = 2 * (size_t)G * D + (size_t)H * E;
+    TFF_REQUIRE(ldp >= C + 2 * (size_t)H && tail_off + (size_t)(taps - 1) * C <= state_row,
+                "gdelta_prep: rows of %zu or state rows of %zu are too short", ldp, state_row);
+    TFF_REQUIRE(2 * G + H + 1 <= 65535, "gdelta_prep: too many heads");
+    if (T == 0) return 0;
+    gdelta_prep_kernel<<<dim3(T, 2 * G + H + 1), 64, 0, (hipStream_t)stream>>>(
+        proj, ldp, wconv, taps, a_log, dt_bias, state, state_row, tail_off, token_req, cu_tokens, state_slots, pre, H, G, D, E);
+    return tff_check_launch("gdelta_prep");
+}
+
+// Sum over the sixteen lanes that share a value channel (neighbours, pairs, quads, halves of the row), the
+// result in all of them; the order of the additions is fixed.
+__device__ __forceinline__ float gd_row16_sum(float v) {
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 8, 64);
+    return v;
+}
+
+// Block: sixteen value channels of one head of one request; a row of sixteen lanes shares a value channel, each
+// lane KPL key channels of it (dim <= 16 KPL; the channels past dim are zero).  The tokens of the portion pass in
+// chunks of sixteen (eight for the widest heads): a chunk's k, q, its sixteen v, beta and decay are fetched into registers while the chunk
+// before is worked through from LDS, so that no token waits for memory; the waves meet at the chunks' borders
+// only.  Per token a lane does 5 KPL multiply-adds and three sums over its row:
+//   a = S^T k, b = S^T q (both of the state before the token), c = k . q;
+//   u = beta (v - g a);   o = g b + c u;   S <- g S + k u.
+template <int KPL>
+__global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
+    const float* __restrict__ pre, const float* __restrict__ proj, size_t ldp, float* __restrict__ state, size_t state_row,
+    size_t tail_off, int taps, const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ state_slots,
+    float* __restrict__ o, int H, int G, int D, int E) {
+    constexpr int DP = 16 * KPL;
+    constexpr int GD_CHUNK = KPL >= 16 ? 8 : 16;           // (two chunks of the widest heads fill LDS otherwise)
+    constexpr int ROWW = 2 * DP + 18;                      // k, q, sixteen v, beta, decay of a token
+    constexpr int NLD = (GD_CHUNK * ROWW + 255) / 256;
+    __shared__ __attribute__((aligned(16))) float lds[2][GD_CHUNK * ROWW];
+    const int h = blockIdx.y, r = blockIdx.z, j0 = blockIdx.x * 16;
+    const int tid = threadIdx.x, s = tid & 15, j = j0 + (tid >> 4);
+    const int C = 2 * G * D + H * E;
+    const size_t ldq = (size_t)C + 2 * H;
+    const int gk = h / (H / G);
+    const int t0 = cu_tokens[r], n = cu_tokens[r + 1] - t0;
+    float* srow = state + (size_t)state_slots[r] * state_row;
+    float S[KPL];
+    float* sp = srow + ((size_t)h * E + min(j, E - 1)) * D + s * KPL;
+#pragma unroll
+    for (int m = 0; m < KPL; ++m) S[m] = (j < E && s * KPL + m < D) ? sp[m] : 0.f;
+
+    float regs[NLD];
+    auto fetch = [&](int first) {
+#pragma unroll
+        for (int x = 0; x < NLD; ++x) {
+            const int e = x * 256 + tid;
+            const int tk = e / ROWW, col = e - tk * ROWW;
+            float v = 0.f;
+            if (tk < GD_CHUNK && first + tk < n) {
+                const float* p = pre + (size_t)(t0 + first + tk) * ldq;
+                if (col < DP) { if (col < D) v = p[(size_t)(G + gk) * D + col]; }
+                else if (col < 2 * DP) { if (col - DP < D) v = p[(size_t)gk * D + col - DP]; }
+                else if (col < 2 * DP + 16) { if (j0 + col - 2 * DP < E) v = p[2 * (size_t)G * D + (size_t)h * E + j0 + col - 2 * DP]; }
+                else v = p[C + (col - 2 * DP - 16) * H + h];
+            }
+            regs[x] = v;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int x = 0; x < NLD; ++x) {
+            const int e = x * 256 + tid;
+            if (e < GD_CHUNK * ROWW) lds[buf][e] = regs[x];
+        }
+    };
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int first = 0; first < n; first += GD_CHUNK) {
+        const bool more = first + GD_CHUNK < n;
+        if (more) fetch(first + GD_CHUNK);
+        const int cnt = min(GD_CHUNK, n - first);
+        for (int tk = 0; tk < cnt; ++tk) {
+            const float* L = lds[buf] + tk * ROWW;
+            float a = 0.f, b = 0.f, c = 0.f, kk[KPL];
+#pragma unroll
+            for (int m = 0; m < KPL; ++m) {
+                kk[m] = L[s * KPL + m];
+                const float qq = L[DP + s * KPL + m];
+                a = fmaf(S[m], kk[m], a);
+                b = fmaf(S[m], qq, b);
+                c = fmaf(kk[m], qq, c);
+            }
+            a = gd_row16_sum(a);
+            b = gd_row16_sum(b);
+            c = gd_row16_sum(c);
+            const float v = L[2 * DP + (tid >> 4)], beta = L[2 * DP + 16], g = L[2 * DP + 17];
+            const float u = beta * (v - g * a);
+#pragma unroll
+            for (int m = 0; m < KPL; ++m) S[m] = fmaf(kk[m], u, g * S[m]);
+            if (s == 0 && j < E) o[(size_t)(t0 + first + tk) * H * E + (size_t)h * E + j] = fmaf(c, u, g * b);
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    if (j < E) {
+#pragma unroll
+        for (int m = 0; m < KPL; ++m)
+            if (s * KPL + m < D) sp[m] = S[m];
+    }
+    // the convolution's last inputs: the head's value channels, and with the first head of a group its q and k
+    if (blockIdx.x == 0 && taps > 1) {
+        float* tail = srow + tail_off;
+        const int own = (h % (H / G) == 0) ? 2 * D : 0;
+        for (int x = tid; x < E + own; x += 256) {
+            const int c = x < E ? 2 * G * D + h * E + x : (x - E < D ? gk * D + x - E : (G + gk) * D + x - E - D);
+            for (int i = 0; i < taps - 1; ++i) {            // ascending: what is read lies behind what was written
+                const int src = n - (taps - 1) + i;
+                tail[(size_t)i * C + c] = src >= 0 ? proj[(size_t)(t0 + src) * ldp + c] : tail[(size_t)(i + n) * C + c];
+            }
+        }
+    }
+}
+
+TFF_API int tff_gdelta_recurrence(const float* pre, const float* proj, size_t ldp, float* state, size_t state_row,
+                                  size_t tail_off, int taps, const int32_t* cu_tokens, const int32_t* state_slots, float* o,
+                                  int R, int H, int G, int D, int E, tff_stream_t stream) {
+    TFF_REQUIRE(pre && proj && state && cu_tokens && state_slots && o, "gdelta_recurrence: null pointer");
+    TFF_REQUIRE(R >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && E > 0 && taps >= 1 && taps <= GD_MAX_TAPS,
+                "gdelta_recurrence: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d taps=%d (dim up to 256, taps up to %d)", H, G, D,
+                E, taps, GD_MAX_TAPS);
+    const size_t C = 2 * (size_t)G * D + (size_t)H * E;
+    TFF_REQUIRE(ldp >= C + 2 * (size_t)H && (size_t)H * E * D <= tail_off && tail_off + (size_t)(taps - 1) * C <= state_row,
+                "gdelta_recurrence: rows of %zu or state rows of %zu are too short", ldp, state_row);
+    TFF_REQUIRE(H <= 65535 && R <= 65535, "gdelta_recurrence: too many heads or requests");
+    if (R == 0) return 0;
+    const dim3 grid((E + 15) / 16, H, R);
+    hipStream_t s = (hipStream_t)stream;
+#define GD_LAUNCH(KPL)                                                                                                     \
+    gdelta_recurrence_kernel<KPL><<<grid, 256, 0, s>>>(pre, proj, ldp, state, state_row, tail_off, taps, cu_tokens, state_slots, \
+                                                       o, H, G, D, E)
+    if (D <= 16) GD_LAUNCH(1);
+    else if (D <= 32) GD_LAUNCH(2);
+    else if (D <= 64) GD_LAUNCH(4);
+    else if (D <= 128) GD_LAUNCH(8);
+    else GD_LAUNCH(16);
+#undef GD_LAUNCH
+    return tff_check_launch("gdelta_recurrence");
+}
+
+// One wave per (token, head): the head's E channels of o are divided by their root mean square, multiplied by
+// w[channel] (one weight for all heads) and by silu(gate), and go to out[t * out_row + h * E + e].
+template <typename TO>
+__global__ __launch_bounds__(256) void head_norm_silu_gate_kernel(const float* __restrict__ o, const float* __restrict__ g,
+                                                                  size_t g_row, const float* __restrict__ w, float eps,
+                                                                  float scale, TO* __restrict__ out, size_t out_row,
+                                                                  int pairs, int H, int E) {
+    const int id = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (id >= pairs) return;
+    const int t = id / H, h = id % H;
+    const float* orow = o + ((size_t)t * H + h) * E;
+    float ss = 0.f;
+    for (int e = lane; e < E; e += 64) ss = fmaf(orow[e], orow[e], ss);
+    ss = wave_sum(ss);
+    const float rr = scale / sqrtf(ss / (float)E + eps);
+    const float* grow = g + (size_t)t * g_row + (size_t)h * E;
+    for (int e = lane; e < E; e += 64)
+        out[(size_t)t * out_row + (size_t)h * E + e] = from_f32<TO>(orow[e] * rr * w[e] * gd_silu(grow[e]));
+}
+
+TFF_API int tff_head_norm_silu_gate(const float* o, const float* g, size_t g_row, const float* w, float eps, float scale,
+                                    void* out, size_t out_row, int T, int H, int E, int out_dtype, tff_stream_t stream) {
+    TFF_REQUIRE(o && g && w && out, "head_norm_silu_gate: null pointer");
+    TFF_REQUIRE(T >= 0 && H > 0 && E > 0 && g_row >= (size_t)H * E && out_row >= (size_t)H * E, "head_norm_silu_gate: bad sizes");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const int pairs = T * H;
+    if (out_dtype == TFF_F32)
+        head_norm_silu_gate_kernel<float><<<(pairs + 3) / 4, 256, 0, s>>>(o, g, g_row, w, eps, scale, (float*)out, out_row, pairs, H, E);
+    else if (out_dtype == TFF_BF16)
+        head_norm_silu_gate_kernel<bf16_t><<<(pairs + 3) / 4, 256, 0, s>>>(o, g, g_row, w, eps, scale, (bf16_t*)out, out_row, pairs, H, E);
+    else
+        return tff_fail("head_norm_silu_gate: unknown dtype %d", out_dtype);
+    return tff_check_launch("head_norm_silu_gate");
+}
+
+// out[t * out_row + h * E + e] = o[t * o_row + h * o_head + e] * sigmoid(g[t * g_row + h * E + e]) * scale
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_gate_heads_kernel(const T* __restrict__ o, size_t o_row, int o_head,
+                                                                 const T* __restrict__ g, size_t g_row, float scale,
+                                                                 T* __restrict__ out, size_t out_row, int HE, int E,
+                                                                 size_t count) {
+    const size_t id = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= count) return;
+    const size_t t = id / HE;
+    const int c = (int)(id - t * HE), h = c / E, e = c - h * E;
+    const float gz = to_f32(g[t * g_row + c]);
+    out[t * out_row + c] = from_f32<T>(to_f32(o[t * o_row + (size_t)h * o_head + e]) * (scale / (1.0f + expf(-gz))));
+}
+
+TFF_API int tff_sigmoid_gate_heads(const void* o, size_t o_row, int o_head, const void* g, size_t g_row, float scale, void* out,
+                                   size_t out_row, int T, int H, int E, int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(o && g && out, "sigmoid_gate_heads: null pointer");
+    TFF_REQUIRE(T >= 0 && H > 0 && E > 0 && o_head >= E && o_row >= (size_t)H * o_head && g_row >= (size_t)H * E &&
+                out_row >= (size_t)H * E, "sigmoid_gate_heads: bad sizes");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t count = (size_t)T * H * E;
+    const unsigned blocks = (unsigned)((count + 255) / 256);
+    if (dtype == TFF_F32)
+        sigmoid_gate_heads_kernel<float><<<blocks, 256, 0, s>>>((const float*)o, o_row, o_head, (const float*)g, g_row, scale,
+                                                                (float*)out, out_row, H * E, E, count);
+    else if (dtype == TFF_BF16)
+        sigmoid_gate_heads_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)o, o_row, o_head, (const bf16_t*)g, g_row, scale,
+                                                                 (bf16_t*)out, out_row, H * E, E, count);
+    else
+        return tff_fail("sigmoid_gate_heads: unknown dtype %d", dtype);
+    return tff_check_launch("sigmoid_gate_heads");
+}

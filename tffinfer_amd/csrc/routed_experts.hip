@@ -147,6 +147,28 @@ TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const floa
     return tff_check_launch("route_topk");
 }
 
+// Experts by a table over the token ids instead of a router: idx[t, k] = table[ids[t], k], each with the weight
+// 1 / top.  An id or an expert outside its range is brought into it (a launch never reads outside a table).
+__global__ __launch_bounds__(256) void route_by_table_kernel(const int32_t* __restrict__ table, const int32_t* __restrict__ ids,
+                                                             int pairs, int V, int top, int E, int32_t* __restrict__ idx,
+                                                             float* __restrict__ wts) {
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= pairs) return;
+    const int t = p / top, k = p - t * top;
+    const int id = min(max(ids[t], 0), V - 1);
+    idx[p] = min(max(table[(size_t)id * top + k], 0), E - 1);
+    wts[p] = 1.0f / (float)top;
+}
+
+TFF_API int tff_route_by_table(const int32_t* table, const int32_t* ids, int T, int V, int top, int E, int32_t* idx,
+                               float* wts, tff_stream_t stream) {
+    TFF_REQUIRE(table && ids && idx && wts, "route_by_table: null pointer");
+    TFF_REQUIRE(T >= 0 && V > 0 && top > 0 && E > 0, "route_by_table: bad sizes T=%d V=%d top=%d E=%d", T, V, top, E);
+    if (T == 0) return 0;
+    route_by_table_kernel<<<(T * top + 255) / 256, 256, 0, (hipStream_t)stream>>>(table, ids, T * top, V, top, E, idx, wts);
+    return tff_check_launch("route_by_table");
+}
+
 #define EX_WAVES 4
 #define EX_PER_WAVE 8      // outputs a wave works through
 
@@ -155,19 +177,27 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
     const T* __restrict__ h, int h_row, const T* __restrict__ Wg, const T* __restrict__ Wu,
     const int32_t* __restrict__ idx, int top, int width, int ff, int ldw, float limit, float act_alpha, float up_offset,
     T* __restrict__ y) {
+    // Wg null: experts without a gate, y = max(Wu h, 0)^2
     const int pair = blockIdx.x;                  // token * top + k
     const int t = pair / top;
     const int e = idx[pair];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const T* hr = h + (size_t)t * h_row;
-    const T* wg = Wg + (size_t)e * ff * ldw;
+    const T* wg = Wg ? Wg + (size_t)e * ff * ldw : nullptr;
     const T* wu = Wu + (size_t)e * ff * ldw;
     const bool vec = sizeof(T) == 2 && width % 8 == 0 && ldw % 8 == 0 && h_row % 8 == 0 && ((uintptr_t)h % 16) == 0 &&
                      ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0;
     const int f0 = (blockIdx.y * EX_WAVES + wv) * EX_PER_WAVE;
     for (int f = f0; f < min(ff, f0 + EX_PER_WAVE); ++f) {
-        float g = row_dot<T>(hr, wg + (size_t)f * ldw, width, lane, vec);
         float u = row_dot<T>(hr, wu + (size_t)f * ldw, width, lane, vec);
+        if (!wg) {
+            if (lane == 0) {
+                u = fmaxf(u, 0.f);
+                y[(size_t)pair * ff + f] = from_f32<T>(u * u);
+            }
+            continue;
+        }
+        float g = row_dot<T>(hr, wg + (size_t)f * ldw, width, lane, vec);
         if (lane == 0) {
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
@@ -199,7 +229,7 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_down_kernel(
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
                                 int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset, void* y,
                                 int dtype, tff_stream_t stream) {
-    TFF_REQUIRE(h && Wg && Wu && idx && y, "experts_gate_up: null pointer");
+    TFF_REQUIRE(h && Wu && idx && y, "experts_gate_up: null pointer");
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && h_row >= width && ldw >= width,
                 "experts_gate_up: bad sizes T=%d top=%d width=%d ff=%d", T, top, width, ff);
     if (T == 0) return 0;
@@ -307,13 +337,15 @@ __device__ __forceinline__ ex_bf16x8 ex_load8(const bf16_t* p, bool ok) {
 // dealt to.
 #define EXT_KSTEP 64
 
-template <bool GATE_UP, int AFR>
+// MODE 0: the down product; 1: gate and up; 2: up alone, y = max(Wu h, 0)^2 (a wave's 32 weight rows are 32 outputs).
+template <int MODE, int AFR>
 __global__ __launch_bounds__(256) void experts_tiles_kernel(
     const bf16_t* __restrict__ a_rows, int a_row, const bf16_t* __restrict__ W0, const bf16_t* __restrict__ W1,
     const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
     const int32_t* __restrict__ num_tiles, const float* __restrict__ wts, int T, int top, int K, int N,
     float limit, float act_alpha, float up_offset, bf16_t* __restrict__ y, float* __restrict__ out, int max_tiles, int col_blocks,
     int ldw) {
+    constexpr bool GATE_UP = MODE == 1;
     constexpr int ROWS = AFR * 16;       // pairs of a tile: 64, or 128 where the experts have many pairs each
     __shared__ __attribute__((aligned(16))) bf16_t lds[2 * AFR * 512];      // two sub-steps of AFR fragments
     // A tile of 64 pairs gives a weight element 128 flops a read: the tiles of one expert must meet
@@ -336,7 +368,7 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
         const int fs = i * 4 + wv, sub = fs / AFR, frag = fs % AFR;
         const int pair = tile_rows[tile * ROWS + frag * 16 + r];
         aok[i] = pair >= 0;
-        asrc[i] = a_rows + (size_t)(GATE_UP ? max(pair, 0) / top : max(pair, 0)) * a_row + sub * 32 + kg * 8;
+        asrc[i] = a_rows + (size_t)(MODE != 0 ? max(pair, 0) / top : max(pair, 0)) * a_row + sub * 32 + kg * 8;
     }
     // the wave's weight rows: two fragments
     const bf16_t* wsrc[2];
@@ -406,6 +438,17 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
                     y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + up_offset));
                 }
             }
+        } else if (MODE == 2) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const float v4[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int n = c0 + j * 16 + kg * 4 + c;
+                    const float u = fmaxf(v4[c], 0.f);
+                    if (pair >= 0 && n < N) y[(size_t)pair * N + n] = (bf16_t)(u * u);
+                }
+            }
         } else {
             const int p = max(pair, 0), t = p / top, k = p - t * top;
             const float w = wts[p];
@@ -434,7 +477,7 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
                                  int ldw_in, int ldw_down, float limit, float act_alpha, float up_offset, int32_t* tile_expert,
                                  int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
                                  tff_stream_t stream) {
-    TFF_REQUIRE(h && Wg && Wu && Wd && idx && wts && tile_expert && tile_rows && num_tiles && y && out,
+    TFF_REQUIRE(h && Wu && Wd && idx && wts && tile_expert && tile_rows && num_tiles && y && out,
                 "experts_by_tiles: null pointer");
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && E <= RT_MAX_E && width > 0 && ff > 0 && h_row >= width,
                 "experts_by_tiles: bad sizes T=%d top=%d E=%d width=%d ff=%d", T, top, E, width, ff);
@@ -455,21 +498,27 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
     experts_sort_kernel<<<1, 1024, 0, s>>>(idx, T * top, E, rows, tile_expert, tile_rows, num_tiles);
     int rc = tff_check_launch("experts_sort");
     if (rc) return rc;
-    const int cb_up = (ff + 63) / 64, cb_down = (width + 127) / 128;
+    const int cb_up = Wg ? (ff + 63) / 64 : (ff + 127) / 128, cb_down = (width + 127) / 128;
 #define EXT_LAUNCH(GU, AFRV, CB, ...) experts_tiles_kernel<GU, AFRV><<<((CB) + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(__VA_ARGS__)
-    if (tall)
-        EXT_LAUNCH(true, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
+    if (!Wg && tall)
+        EXT_LAUNCH(2, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wu, nullptr, tile_expert, tile_rows,
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+    else if (!Wg)
+        EXT_LAUNCH(2, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wu, nullptr, tile_expert, tile_rows,
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+    else if (tall)
+        EXT_LAUNCH(1, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
                    num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
     else
-        EXT_LAUNCH(true, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
+        EXT_LAUNCH(1, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
                    num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
     rc = tff_check_launch("experts_gate_up_tiles");
     if (rc) return rc;
     if (tall)
-        EXT_LAUNCH(false, 8, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
+        EXT_LAUNCH(0, 8, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
                    T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down);
     else
-        EXT_LAUNCH(false, 4, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
+        EXT_LAUNCH(0, 4, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
                    T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down);
 #undef EXT_LAUNCH
     return tff_check_launch("experts_down_tiles");

@@ -311,6 +311,41 @@ TFF_API int tff_head_norm_gate(const float* o, const float* g, size_t g_row, con
                                int H, int D, int out_dtype, tff_stream_t stream);
 TFF_API int tff_tanh(const float* in, void* out, size_t count, int out_dtype, tff_stream_t stream);
 
+// ---- the gated delta rule (gated_delta.hip) ----
+// proj float32 [T, >= C + 2 H] (rows ldp apart): q [G x D], k [G x D], v [H x E] (C channels), b [H], a [H].
+// pre float32 [T, C + 2 H]: q, k, v after the causal convolution over time (wconv float32 [C, taps], the last tap
+// the token's own) and silu, q and k as unit vectors per head (q times D^(-1/2)); beta = sigmoid(b);
+// decay = exp(-exp(a_log) softplus(a + dt_bias)).  The inputs before a portion's first token come from the
+// request's state row at tail_off: [taps - 1][C], oldest first.
+TFF_API int tff_gdelta_prep(const float* proj, size_t ldp, const float* wconv, int taps, const float* a_log,
+                            const float* dt_bias, const float* state, size_t state_row, size_t tail_off,
+                            const int32_t* token_req, const int32_t* cu_tokens, const int32_t* state_slots, float* pre,
+                            int T, int H, int G, int D, int E, tff_stream_t stream);
+// Per request (cu_tokens, state_slots) and head h (keys and queries of head h / (H / G)), S^T [E, D] at the start of
+// the state row: S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  o float32 [T, H * E].  The
+// portion's last taps - 1 rows of proj's channels are left at tail_off of the state row.
+TFF_API int tff_gdelta_recurrence(const float* pre, const float* proj, size_t ldp, float* state, size_t state_row,
+                                  size_t tail_off, int taps, const int32_t* cu_tokens, const int32_t* state_slots, float* o,
+                                  int R, int H, int G, int D, int E, tff_stream_t stream);
+// out[t * out_row + h * E + e] = o[t, h, e] / sqrt(mean over e of o^2 + eps) * w[e] * silu(g[t * g_row + h * E + e]) * scale
+TFF_API int tff_head_norm_silu_gate(const float* o, const float* g, size_t g_row, const float* w, float eps, float scale,
+                                    void* out, size_t out_row, int T, int H, int E, int out_dtype, tff_stream_t stream);
+// out[t * out_row + h * E + e] = o[t * o_row + h * o_head + e] * sigmoid(g[t * g_row + h * E + e]) * scale
+TFF_API int tff_sigmoid_gate_heads(const void* o, size_t o_row, int o_head, const void* g, size_t g_row, float scale, void* out,
+                                   size_t out_row, int T, int H, int E, int dtype, tff_stream_t stream);
+
+// ---- two norms of one sum, the cap on the logits (pair_norm.hip) ----
+// v = resid + planes of d0 + planes of d1 + bias (each optional); resid <- v unless rows picks rows;
+// out1 = rmsnorm(v) * w1, out2 = rmsnorm(v) * w2 (w2 optional).
+TFF_API int tff_add_rmsnorm_pair(float* resid, const float* d0, int planes0, size_t plane0, const float* d1, int planes1,
+                                 size_t plane1, const float* bias, const float* w1, const float* w2, float eps, void* out1,
+                                 void* out2, const int32_t* rows, int n, int W, int out_dtype, tff_stream_t stream);
+// z <- cap * tanh(z / cap), in place.
+TFF_API int tff_softcap(float* z, size_t count, float cap, tff_stream_t stream);
+// idx[t, :] = table[ids[t], :] (int32 [V, top]), wts[t, :] = 1 / top: experts by a table over the token ids.
+TFF_API int tff_route_by_table(const int32_t* table, const int32_t* ids, int T, int V, int top, int E, int32_t* idx,
+                               float* wts, tff_stream_t stream);
+
 // ---- attention whose heads exchange their scores (mixed_attention.hip) ----
 TFF_API int tff_qk_bias_norm_store(const float* qk, size_t row, const float* qb, const float* kb, float eps, void* q_out,
                                    void* k_cache, void* v_cache, const int32_t* slot_mapping, int page_size, int T, int H,

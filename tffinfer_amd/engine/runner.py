@@ -24,7 +24,7 @@ class StepError(ValueError):
 
 class LayerContext:
     """What a part sees during one layer call of one step."""
-    __slots__ = ("ops", "act_dtype", "batch", "max_positions", "kv", "state", "call_index")
+    __slots__ = ("ops", "act_dtype", "batch", "max_positions", "kv", "state", "call_index", "stream_offset")
 
     def __init__(self, ops, act_dtype, batch, max_positions):
         self.ops = ops
@@ -34,6 +34,7 @@ class LayerContext:
         self.kv = None
         self.state = None
         self.call_index = -1
+        self.stream_offset = None       # float32 [hidden]: a row the run order adds to the stream before this call
 
 
 class StepContext(LayerContext):

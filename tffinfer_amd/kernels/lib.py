@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 30
+ABI_VERSION = 31
 
 
 class KernelLibraryError(RuntimeError):
@@ -61,6 +61,13 @@ _SIGNATURES = {
     "tff_wkv_recurrence": [_P, _P, _P, _P, _Z, _P, _P, _P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _Z, _I, _P],
     "tff_head_norm_gate": [_P, _P, _Z, _P, _F, _P, _I, _I, _I, _I, _P],
     "tff_tanh": [_P, _P, _Z, _I, _P],
+    "tff_gdelta_prep": [_P, _Z, _P, _I, _P, _P, _P, _Z, _Z, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "tff_gdelta_recurrence": [_P, _P, _Z, _P, _Z, _Z, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "tff_head_norm_silu_gate": [_P, _P, _Z, _P, _F, _F, _P, _Z, _I, _I, _I, _I, _P],
+    "tff_sigmoid_gate_heads": [_P, _Z, _I, _P, _Z, _F, _P, _Z, _I, _I, _I, _I, _P],
+    "tff_add_rmsnorm_pair": [_P, _P, _I, _Z, _P, _I, _Z, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P],
+    "tff_softcap": [_P, _Z, _F, _P],
+    "tff_route_by_table": [_P, _P, _I, _I, _I, _I, _P, _P, _P],
     "tff_qk_bias_norm_store": [_P, _Z, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "tff_mixed_attention_supported": [_I, _I, _I],
     "tff_mixed_attention": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _F, _F, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P],

@@ -215,6 +215,11 @@ class ScaledRows:
         return add_rmsnorm(self.resid, None, self.weight, self.eps, self.x.dtype)
 
 
+def _as_tensor_terms(t) -> torch.Tensor:
+    parts = [as_tensor(x) for x in t.terms]
+    return parts[0] if len(parts) == 1 else parts[0] + parts[1]
+
+
 def as_tensor(t) -> torch.Tensor:
     """Whatever ``linear`` or ``add_rmsnorm`` returned, as a plain tensor: a
     product that has not run is run, partial sums [S, T, H] are added up in
@@ -223,6 +228,8 @@ def as_tensor(t) -> torch.Tensor:
         return t.run()
     if isinstance(t, ScaledRows):
         return t.materialize()
+    if isinstance(t, PendingTerms):
+        return _as_tensor_terms(t)
     if isinstance(t, torch.Tensor) and t.dim() == 3:
         acc = t[0].clone()
         for part in t[1:]:
@@ -255,6 +262,10 @@ def add_rmsnorm(resid: torch.Tensor, delta, weight: torch.Tensor, eps: float,
     [S, T, H] of partial sums, which are added up first, in order, or a
     product that has not run.  ``for_linear``: the result goes to ``linear``
     and nowhere else, so it may be a :class:`ScaledRows`."""
+    if isinstance(delta, PendingTerms):
+        if out is not None:
+            raise _lib.KernelError("add_rmsnorm: several pending terms and a given result do not go together")
+        return add_rmsnorm_pair(resid, delta, None, weight, None, eps, out_dtype, rows=rows)[0]
     _req(resid, "add_rmsnorm resid", torch.float32, 2)
     H = resid.shape[1]
     _req(weight, "add_rmsnorm weight", torch.float32, 1)
@@ -1068,6 +1079,7 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
                    by_tiles: bool | None = None, up_offset: float = 1.0) -> torch.Tensor:
     """The weighted sum of each token's chosen experts: y = g sigmoid(act_alpha g) (u + up_offset) with
     g = min(Wg h, limit), u = clamp(Wu h, -limit, limit); out = sum_k wts[:, k] Wd y.
+    ``w_gate`` None: experts without a gate, y = max(Wu h, 0)^2.
     ``w_gate``, ``w_up`` [E, ff, >= width], ``w_down`` [E, width, >= ff] of h's type (the last
     dimension may be wider than what is multiplied: see :func:`pad_expert_rows`).  float32
     [T, width], or (many tokens in bfloat16, ``by_tiles``) [top, T, width]: the terms of the sum
@@ -1075,11 +1087,13 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
     _req(h, "routed_experts h", ndim=2)
     T, width = h.shape
     for w, nm in ((w_gate, "gate"), (w_up, "up"), (w_down, "down")):
-        _req(w, f"experts {nm}", h.dtype, 3)
-    E, ff, ld_in = w_gate.shape
+        if w is not None or nm != "gate":
+            _req(w, f"experts {nm}", h.dtype, 3)
+    E, ff, ld_in = w_up.shape
     ld_down = w_down.shape[2]
-    if ld_in < width or tuple(w_up.shape) != (E, ff, ld_in) or tuple(w_down.shape[:2]) != (E, width) or ld_down < ff:
-        raise _lib.KernelError(f"routed_experts: weights {tuple(w_gate.shape)}, {tuple(w_up.shape)}, "
+    if ld_in < width or (w_gate is not None and tuple(w_gate.shape) != (E, ff, ld_in)) \
+            or tuple(w_down.shape[:2]) != (E, width) or ld_down < ff:
+        raise _lib.KernelError(f"routed_experts: weights {w_gate is not None and tuple(w_gate.shape)}, {tuple(w_up.shape)}, "
                                f"{tuple(w_down.shape)} for rows of {width}")
     _req(idx, "experts idx", torch.int32, 2)
     _req(wts, "experts weights", torch.float32, 2)
@@ -1097,11 +1111,11 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
         tables = torch.empty(129 * max_tiles + 1, dtype=torch.int32, device=h.device)
         out = torch.empty(top, T, width, dtype=torch.float32, device=h.device)
         _lib.check(L.tff_experts_by_tiles(
-            h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(),
+            h.data_ptr(), width, _ptr(w_gate), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(),
             T, top, E, width, ff, ld_in, ld_down, float(limit), float(act_alpha), float(up_offset), tables.data_ptr(), tables[max_tiles:].data_ptr(),
             tables[129 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), _stream()))
         return out if top > 1 else out[0]
-    _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), idx.data_ptr(), T, top, E,
+    _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, _ptr(w_gate), w_up.data_ptr(), idx.data_ptr(), T, top, E,
                                      width, ff, ld_in, float(limit), float(act_alpha), float(up_offset), y.data_ptr(), dtype_code(h.dtype),
                                      _stream()))
     out = torch.empty(T, width, dtype=torch.float32, device=h.device)
@@ -1372,6 +1386,158 @@ def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: f
                                      rows, _ptr(mix), float(scale), float(softcap), int(window), int(keep_first),
                                      1 if sink else 0, out.data_ptr(), T, H, G, D, kv.page_size, splits, per, _ptr(ws),
                                      dtype_code(dt), _stream()))
+    return out
+
+
+class PendingTerms:
+    """Several terms that a block has not added to the residual stream yet (a layer whose mixer and
+    feed-forward read the same rows leaves two); each is what a mixer or feed-forward may return:
+    a tensor, a stack of partial sums or a product that has not run.  ``add_rmsnorm_pair`` and
+    ``add_rmsnorm`` take them; ``as_tensor`` adds them up."""
+
+    def __init__(self, terms):
+        self.terms = [t for t in terms if t is not None]
+        if len(self.terms) > 2:
+            raise _lib.KernelError("pending terms: at most two")
+
+
+def _planes_of(delta, shape, what: str):
+    """(tensor or None, planes, plane stride) of a pending term for a kernel that adds planes up."""
+    if delta is None:
+        return None, 0, 0
+    if isinstance(delta, PendingProduct):
+        delta = delta.run()
+    _req(delta, what, torch.float32, 3 if delta.dim() == 3 else 2)
+    if tuple(delta.shape[-2:]) != tuple(shape):
+        raise _lib.KernelError(f"{what}: {tuple(delta.shape)} does not match the stream {tuple(shape)}")
+    if delta.dim() == 3:
+        return delta, delta.shape[0], delta.stride(0)
+    return delta, 1, 0
+
+
+def add_rmsnorm_pair(resid: torch.Tensor, delta, bias: torch.Tensor | None, w1: torch.Tensor,
+                     w2: torch.Tensor | None, eps: float, out_dtype: torch.dtype,
+                     rows: torch.Tensor | None = None):
+    """``resid += terms + bias`` (``delta``: None, one pending term or :class:`PendingTerms`; ``bias``
+    float32 [H] or None) and two RMS norms of the sum, one with each weight (``w2`` None: one);
+    with ``rows`` the norms of those rows only, ``resid`` untouched.  Returns (out1, out2 or None)."""
+    _req(resid, "add_rmsnorm_pair resid", torch.float32, 2)
+    H = resid.shape[1]
+    for w, nm in ((w1, "first weight"), (w2, "second weight"), (bias, "bias")):
+        if w is not None:
+            _req(w, f"add_rmsnorm_pair {nm}", torch.float32, 1)
+            if w.numel() != H:
+                raise _lib.KernelError(f"add_rmsnorm_pair: {nm} has {w.numel()} elements, rows have {H}")
+    terms = delta.terms if isinstance(delta, PendingTerms) else ([] if delta is None else [delta])
+    d = [_planes_of(t, resid.shape, "add_rmsnorm_pair term") for t in terms] + [(None, 0, 0)] * 2
+    if rows is not None:
+        _req(rows, "add_rmsnorm_pair rows", torch.int32, 1)
+        n = rows.numel()
+    else:
+        n = resid.shape[0]
+    out1 = torch.empty(n, H, dtype=out_dtype, device=resid.device)
+    out2 = torch.empty(n, H, dtype=out_dtype, device=resid.device) if w2 is not None else None
+    _lib.check(_lib.load().tff_add_rmsnorm_pair(
+        resid.data_ptr(), _ptr(d[0][0]), d[0][1], d[0][2], _ptr(d[1][0]), d[1][1], d[1][2], _ptr(bias), w1.data_ptr(),
+        _ptr(w2), float(eps), out1.data_ptr(), _ptr(out2), _ptr(rows), n, H, dtype_code(out_dtype), _stream()))
+    return out1, out2
+
+
+def softcap_(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """z <- cap * tanh(z / cap) in place on float32."""
+    _req(z, "softcap", torch.float32)
+    _lib.check(_lib.load().tff_softcap(z.data_ptr(), z.numel(), float(cap), _stream()))
+    return z
+
+
+def route_by_table(table: torch.Tensor, token_ids: torch.Tensor, num_experts: int):
+    """Experts by a table over the token ids (int32 [vocab, top]): (int32 [T, top], float32 [T, top] = 1 / top)."""
+    _req(table, "route_by_table table", torch.int32, 2)
+    _req(token_ids, "route_by_table ids", torch.int32, 1)
+    T, (V, top) = token_ids.numel(), table.shape
+    idx = torch.empty(T, top, dtype=torch.int32, device=table.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=table.device)
+    _lib.check(_lib.load().tff_route_by_table(table.data_ptr(), token_ids.data_ptr(), T, V, top, int(num_experts),
+                                              idx.data_ptr(), wts.data_ptr(), _stream()))
+    return idx, wts
+
+
+def _rows2(t: torch.Tensor, name: str, dtype, cols: int):
+    """A GPU matrix with unit inner stride (rows may be strided) of at least ``cols`` columns; its row stride."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.dtype != dtype \
+            or t.shape[1] < cols:
+        raise _lib.KernelError(f"{name}: expected a GPU matrix of {dtype} with unit inner stride and {cols} columns or more")
+    return t.stride(0) if t.shape[0] > 1 else t.shape[1]
+
+
+def gated_delta(proj: torch.Tensor, conv_w: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                state: torch.Tensor, batch, H: int, G: int, D: int, E: int) -> torch.Tensor:
+    """The gated delta rule over the step's tokens.  ``proj`` float32 [T, >= C + 2 H]: the projections q [G, D],
+    k [G, D], v [H, E] (C = 2 G D + H E channels), b [H], a [H]; ``conv_w`` float32 [C, taps]; ``state`` float32
+    [slots, >= H E D + (taps - 1) C]: per request the heads' matrices and the convolution's last inputs.
+    q, k, v pass the causal convolution and silu; q, k become unit vectors per head (q times D^(-1/2));
+    beta = sigmoid(b); decay = exp(-exp(a_log) softplus(a + dt_bias)); per head (keys and queries of head
+    h // (H / G)): S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Returns o float32 [T, H E]."""
+    C = 2 * G * D + H * E
+    T = proj.shape[0]
+    ldp = _rows2(proj, "gated_delta proj", torch.float32, C + 2 * H)
+    _req(conv_w, "gated_delta conv", torch.float32, 2)
+    _req(a_log, "gated_delta a_log", torch.float32, 1)
+    _req(dt_bias, "gated_delta dt_bias", torch.float32, 1)
+    taps = conv_w.shape[1]
+    if conv_w.shape[0] != C or a_log.numel() != H or dt_bias.numel() != H:
+        raise _lib.KernelError(f"gated_delta: conv {tuple(conv_w.shape)}, {a_log.numel()} / {dt_bias.numel()} decay terms "
+                               f"for {C} channels and {H} heads")
+    row = _state_rows(state, "gated_delta state")
+    tail = H * E * D
+    if tail + (taps - 1) * C > row:
+        raise _lib.KernelError(f"gated_delta: state rows of {row} do not hold {H} x {E} x {D} and {taps - 1} x {C}")
+    if batch.num_tokens != T:
+        raise _lib.KernelError(f"gated_delta: {T} rows for a step of {batch.num_tokens} tokens")
+    pre = torch.empty(T, C + 2 * H, dtype=torch.float32, device=proj.device)
+    o = torch.empty(T, H * E, dtype=torch.float32, device=proj.device)
+    if T == 0:
+        return o
+    L = _lib.load()
+    stream = _stream()
+    _lib.check(L.tff_gdelta_prep(proj.data_ptr(), ldp, conv_w.data_ptr(), taps, a_log.data_ptr(), dt_bias.data_ptr(),
+                                 state.data_ptr(), row, tail, batch.token_req.data_ptr(), batch.cu_tokens.data_ptr(),
+                                 batch.state_slots.data_ptr(), pre.data_ptr(), T, H, G, D, E, stream))
+    _lib.check(L.tff_gdelta_recurrence(pre.data_ptr(), proj.data_ptr(), ldp, state.data_ptr(), row, tail, taps,
+                                       batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), o.data_ptr(),
+                                       batch.num_reqs, H, G, D, E, stream))
+    return o
+
+
+def head_norm_silu_gate(o: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, eps: float, H: int, E: int,
+                        out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """``out[:, h E + e] = o[:, h, e] / sqrt(mean over the head of o^2 + eps) * weight[e] * silu(g) * scale`` for o
+    float32 [T, H E], g float32 [T, >= H E] and out [T, >= H E] (rows of g and out may be strided)."""
+    _req(o, "head_norm_silu_gate o", torch.float32, 2)
+    _req(weight, "head_norm_silu_gate weight", torch.float32, 1)
+    T = o.shape[0]
+    if o.shape[1] != H * E or weight.numel() != E or g.shape[0] != T or out.shape[0] != T:
+        raise _lib.KernelError("head_norm_silu_gate: o must be [T, heads * vdim], the weight [vdim]")
+    g_row = _rows2(g, "head_norm_silu_gate g", torch.float32, H * E)
+    out_row = _rows2(out, "head_norm_silu_gate out", out.dtype, H * E)
+    _lib.check(_lib.load().tff_head_norm_silu_gate(o.data_ptr(), g.data_ptr(), g_row, weight.data_ptr(), float(eps),
+                                                   float(scale), out.data_ptr(), out_row, T, H, E, dtype_code(out.dtype),
+                                                   _stream()))
+    return out
+
+
+def sigmoid_gate_heads(o: torch.Tensor, o_head: int, g: torch.Tensor, H: int, E: int, out: torch.Tensor,
+                       scale: float = 1.0) -> torch.Tensor:
+    """``out[:, h E + e] = o[:, h o_head + e] * sigmoid(g[:, h E + e]) * scale``: the first E elements of every head
+    of o (heads ``o_head`` apart) times a gate; rows of all three may be strided."""
+    T = o.shape[0]
+    o_row = _rows2(o, "sigmoid_gate_heads o", o.dtype, H * o_head)
+    g_row = _rows2(g, "sigmoid_gate_heads g", o.dtype, H * E)
+    out_row = _rows2(out, "sigmoid_gate_heads out", o.dtype, H * E)
+    if g.shape[0] != T or out.shape[0] != T or o_head < E:
+        raise _lib.KernelError("sigmoid_gate_heads: o, g and out must have one row per token")
+    _lib.check(_lib.load().tff_sigmoid_gate_heads(o.data_ptr(), o_row, int(o_head), g.data_ptr(), g_row, float(scale),
+                                                  out.data_ptr(), out_row, T, H, E, dtype_code(o.dtype), _stream()))
     return out
 
 

@@ -26,6 +26,8 @@ class TensorNames:
     layer: str = "model.layers.{i}"
     final_norm: str = "model.norm"
     head: str = "lm_head"
+    #: the table of vectors the run order adds to the stream, for architectures that have one
+    stream_offsets: str = "stream_offsets"
     #: the block's children by the name the files use
     children: dict = field(default_factory=dict)
     #: tensors a file may hold that the model has no use for
@@ -48,6 +50,27 @@ def _leaves(prefix: str, part: Part, rename: dict):
         yield from _leaves(f"{prefix}.{rename.get(child_name, child_name)}", child, rename)
 
 
+class StreamOffsets(Part):
+    """A table [rows, hidden] of vectors that the run order adds to the residual stream before
+    certain layer calls (``LayerCall.offset`` names the row); float32."""
+
+    graph_safe = True
+
+    def __init__(self, rows: int, hidden_size: int):
+        self.rows = int(rows)
+        self.hidden_size = int(hidden_size)
+        self.weight = None
+
+    def weight_specs(self):
+        return {"weight": WeightSpec((self.rows, self.hidden_size), "vector")}
+
+    def load_weights(self, weights, dtype, device):
+        self.weight = weights["weight"].to(torch.float32).contiguous().to(device)
+
+    def row(self, i: int) -> torch.Tensor:
+        return self.weight[i]
+
+
 class DecoderModel:
     def __init__(self, config: ModelConfig, names: TensorNames):
         self.config = config
@@ -55,7 +78,11 @@ class DecoderModel:
         self.dtype = None
         self.device = None
         H, V = config.hidden_size, config.vocab_size
-        self.embedding = Embedding(V, H, scale=getattr(config, "embedding_scale", 1.0))
+        emb_norm = config.embedding_norm_spec() if hasattr(config, "embedding_norm_spec") else None
+        self.embedding = Embedding(V, H, scale=getattr(config, "embedding_scale", 1.0),
+                                   norm=NORMS.build(emb_norm) if emb_norm is not None else None)
+        n_off = config.stream_offset_rows() if hasattr(config, "stream_offset_rows") else 0
+        self.stream_offsets = StreamOffsets(n_off, H) if n_off else None
         self.blocks = []
         for spec in config.layer_specs():
             mixer = MIXERS.build(spec.mixer)
@@ -74,12 +101,18 @@ class DecoderModel:
         for call in self.schedule:
             if not 0 <= call.layer < len(self.blocks):
                 raise ValueError(f"layer schedule names layer {call.layer}, the model has {len(self.blocks)}")
+            if call.offset >= (self.stream_offsets.rows if self.stream_offsets else 0):
+                raise ValueError(f"layer schedule names stream offset {call.offset}, the model has "
+                                 f"{self.stream_offsets.rows if self.stream_offsets else 0}")
         self.final_norm = NORMS.build(config.final_norm_spec())
-        self.head = OutputHead(V, H, self.embedding if config.tie_word_embeddings else None)
+        self.head = OutputHead(V, H, self.embedding if config.tie_word_embeddings else None,
+                               softcap=getattr(config, "logit_softcap", None))
 
     # ---- weights ---------------------------------------------------------
     def _weighted_parts(self):
-        yield self.names.embedding, self.embedding
+        yield from _leaves(self.names.embedding, self.embedding, {})
+        if self.stream_offsets is not None:
+            yield self.names.stream_offsets, self.stream_offsets
         for i, block in zip(self.layer_numbers, self.blocks):
             yield from _leaves(self.names.layer.format(i=i), block, self.names.children)
         yield self.names.final_norm, self.final_norm
@@ -137,7 +170,7 @@ class DecoderModel:
 
     def _item_graph_safe(self, item) -> bool:
         if item == "embed":
-            parts = [self.embedding]
+            parts = [p for _, p in _leaves("", self.embedding, {})]
         elif item == "finish":
             parts = [self.final_norm, self.head]
         else:
@@ -198,5 +231,14 @@ class DecoderModel:
                     logits = self.head.forward(ctx, y)
             else:
                 call = self.schedule[it]
-                pending = self.blocks[call.layer].forward(ctx.for_call(it), resid, pending)
+                block, c = self.blocks[call.layer], ctx.for_call(it)
+                if call.offset >= 0:
+                    if getattr(block, "takes_stream_offset", False):
+                        c.stream_offset = self.stream_offsets.row(call.offset)
+                    else:       # a block that knows nothing of offsets finds them in the stream
+                        if pending is not None:
+                            resid += ctx.ops.as_tensor(pending)
+                            pending = None
+                        resid += self.stream_offsets.row(call.offset)
+                pending = block.forward(c, resid, pending)
         return resid, pending, logits

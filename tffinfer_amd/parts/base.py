@@ -33,10 +33,12 @@ class WeightSpec:
     ``unit_interval`` U(0, 1), ``decay_log`` U(-3, 0.5) (z of a decay exp(-exp(z))), ``depth_coef``
     N(0, 0.2) with 1 added to the last element.  A dimension of ``shape`` may be None: the
     tensor itself gives that size (random weights then need it from the part's arguments).
-    ``optional``: a file may leave the tensor out, and the part then does without it."""
+    ``optional``: a file may leave the tensor out, and the part then does without it.
+    ``index_table``: an integer table (int32) whose rows hold different numbers below ``bound``."""
     shape: tuple
     init: str = "matrix"
     optional: bool = False
+    bound: int = 0
 
 
 @dataclass(frozen=True)

@@ -170,3 +170,42 @@ class OutputNormBlock(Block):
             h = resid if h is None else h
         ctx.batch._normed_rows = (resid, ctx.call_index, h)
         return None
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """x <- x + (mixer(norm1(x)) + ffn(norm2(x))): both sublayers read the same x, each through a norm
+    of its own.  The two outputs stay pending for the block after it (or the model's last norm), whose
+    first kernel adds them to the stream and forms its two norms in one pass; a row the run order asks to
+    be added to the stream before this call (``ctx.stream_offset``) rides in the same pass.  A layer
+    without a feed-forward has no second norm."""
+
+    graph_safe = True
+    #: the block adds ``ctx.stream_offset`` to the stream itself
+    takes_stream_offset = True
+
+    def __init__(self, mixer, feed_forward, make_norm):
+        self.norm1 = make_norm()
+        self.mixer = mixer
+        self.norm2 = make_norm()
+        self.feed_forward = feed_forward
+        self.has_ffn = not getattr(feed_forward, "is_none", False)
+        if not self.has_ffn:
+            self.norm2.optional = True
+        for n in (self.norm1, self.norm2):
+            if not hasattr(n, "weight") or not hasattr(n, "eps") or getattr(n, "groups", 1) != 1:
+                from ..config.base import ConfigError
+                raise ConfigError("parallel block: its norms are RMS norms over the whole row")
+
+    def children(self):
+        return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
+                "feed_forward": self.feed_forward}
+
+    def forward(self, ctx, resid, pending):
+        ops = ctx.ops
+        h1, h2 = ops.add_rmsnorm_pair(resid, pending, getattr(ctx, "stream_offset", None), self.norm1.weight,
+                                      self.norm2.weight if self.has_ffn else None, self.norm1.eps, ctx.act_dtype)
+        a = self.mixer.forward(ctx, h1)
+        if not self.has_ffn:
+            return a
+        return ops.PendingTerms([a, self.feed_forward.forward(ctx, h2)])

@@ -186,3 +186,58 @@ class RoutedExperts(FeedForward):
             idx, wts = ops.route_topk(x, self.router, self.correction, self.top, softmax=self.router_softmax)
         return ops.routed_experts(x, self.w_gate, self.w_up, self.w_down, idx, wts, self.limit, self.act_alpha,
                                   up_offset=self.up_offset)
+
+
+@register_feed_forward("table_experts")
+class TableExperts(FeedForward):
+    """``num_experts`` small feed-forwards without a gate, f_e = Wd max(Wu z, 0)^2, of which every token
+    uses ``top``: a table over the vocabulary (int32 [vocab, top], the entries of a row differ) names them
+    by the token's id, and each counts 1 / top.  There is no router.  The experts' matrices lie stacked,
+    [experts, out, in], as those of ``RoutedExperts``, and run on the same kernels."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, vocab_size: int):
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.num_experts = int(num_experts)
+        self.top = int(top)
+        self.vocab_size = int(vocab_size)
+        if not 0 < self.top <= self.num_experts:
+            from ..config.base import ConfigError
+            raise ConfigError(f"table experts: top={self.top} of {self.num_experts} experts")
+        self.w_up = self.w_down = self.table = None
+
+    def weight_specs(self):
+        H, I = self.hidden_size, self.intermediate_size
+        specs = {"table": WeightSpec((self.vocab_size, self.top), "index_table", bound=self.num_experts)}
+        for e in range(self.num_experts):
+            specs[f"e{e}.up"] = WeightSpec((I, H))
+            specs[f"e{e}.down"] = WeightSpec((H, I))
+        return specs
+
+    def active_matrix_elements(self) -> int:
+        return self.top * 2 * self.hidden_size * self.intermediate_size
+
+    def streamed_matrix_elements(self, rows: int) -> int:
+        return min(self.num_experts, rows * self.top) * 2 * self.hidden_size * self.intermediate_size
+
+    def load_weights(self, weights, dtype, device):
+        from ..kernels.ops import pad_expert_rows
+        E = self.num_experts
+
+        def stack(which):
+            return pad_expert_rows(torch.stack([weights[f"e{e}.{which}"].to(dtype) for e in range(E)], 0)).to(device)
+
+        self.w_up, self.w_down = stack("up"), stack("down")
+        table = weights["table"].to(torch.int32)
+        if int(table.min()) < 0 or int(table.max()) >= E:
+            from ..config.base import ConfigError
+            raise ConfigError(f"table experts: the table names experts outside 0 .. {E - 1}")
+        self.table = table.contiguous().to(device)
+
+    def forward(self, ctx, x):
+        ops = ctx.ops
+        x = ops.as_tensor(x)
+        idx, wts = ops.route_by_table(self.table, ctx.batch.token_ids, self.num_experts)
+        return ops.routed_experts(x, None, self.w_up, self.w_down, idx, wts, float("inf"), 1.0, up_offset=0.0)

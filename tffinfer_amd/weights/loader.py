@@ -23,11 +23,12 @@ class WeightError(ValueError):
         for name, want, got in self.wrong_shape:
             lines.append(f"  wrong shape: {name}: expected {list(want)}, found {list(got)}")
         for name, got in self.wrong_dtype:
-            lines.append(f"  unsupported type: {name}: {got} (float32, bfloat16 or float16)")
+            lines.append(f"  unsupported type: {name}: {got} (float32, bfloat16 or float16; integers for a table of indices)")
         super().__init__("\n".join(lines))
 
 
 _FLOATS = (torch.float32, torch.bfloat16, torch.float16)
+_INTS = (torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8)      # (a table of indices)
 
 
 def check_weights(expected: dict[str, WeightSpec], found: dict[str, torch.Tensor],
@@ -41,7 +42,8 @@ def check_weights(expected: dict[str, WeightSpec], found: dict[str, torch.Tensor
 
     wrong_shape = [(n, expected[n].shape, tuple(found[n].shape)) for n in expected
                    if n in found and not fits(tuple(expected[n].shape), tuple(found[n].shape))]
-    wrong_dtype = [(n, found[n].dtype) for n in expected if n in found and found[n].dtype not in _FLOATS]
+    wrong_dtype = [(n, found[n].dtype) for n in expected if n in found and
+                   found[n].dtype not in (_INTS if expected[n].init == "index_table" else _FLOATS)]
     if missing or unexpected or wrong_shape or wrong_dtype:
         raise WeightError(sorted(missing), sorted(unexpected), wrong_shape, wrong_dtype, where)
 

@@ -13,8 +13,8 @@ from .safetensors_io import save_file
 MATRIX_STD = 0.02
 NORM_STD = 0.1
 VECTOR_STD = 0.5
-#: laws whose tensors are kept in float32 whatever the matrices are stored in
-FLOAT32_INITS = ("norm", "norm_offset", "vector", "unit_interval", "decay_log", "depth_coef")
+#: laws whose tensors are kept as drawn (float32, or int32 for a table of indices) whatever the matrices are stored in
+FLOAT32_INITS = ("norm", "norm_offset", "vector", "unit_interval", "decay_log", "depth_coef", "index_table")
 
 
 def tensor_seed(seed: int, name: str) -> int:
@@ -32,6 +32,13 @@ def random_tensor(spec: WeightSpec, seed: int, name: str, device="cpu") -> torch
     if any(n is None for n in spec.shape):
         raise ValueError(f"random weights for '{name}': its shape {spec.shape} leaves a size open; "
                          "give the part that size as an argument")
+    if spec.init == "index_table":
+        # int32: every row the first numbers of a random order of 0 .. bound - 1
+        rows, per = spec.shape
+        if not 0 < per <= spec.bound:
+            raise ValueError(f"random weights for '{name}': rows of {per} different numbers below {spec.bound}")
+        order = torch.rand(rows, spec.bound, generator=g, dtype=torch.float32, device=device).argsort(1)
+        return order[:, :per].to(torch.int32).contiguous()
     if spec.init in ("unit_interval", "decay_log"):
         x = torch.rand(spec.shape, generator=g, dtype=torch.float32, device=device)
         return x if spec.init == "unit_interval" else 3.5 * x - 3.0
