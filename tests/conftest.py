@@ -37,6 +37,14 @@ def netovik_dirs(tmp_path_factory):
     return {name: make_netovik_dir(str(base / name), cfg, seed) for name, (cfg, seed) in NETOVIK_CONFIGS.items()}
 
 
+@pytest.fixture(scope="session")
+def sipilorn_dirs(tmp_path_factory):
+    """Model folders of the tiny Sipilorn configurations (sharpened weights), once per session."""
+    from sipilorn_models import SIPILORN_CONFIGS, make_sipilorn_dir
+    base = tmp_path_factory.mktemp("sipilorn")
+    return {name: make_sipilorn_dir(str(base / name), cfg, seed) for name, (cfg, seed) in SIPILORN_CONFIGS.items()}
+
+
 @pytest.fixture(autouse=True)
 def _seeded():
     """Every test draws the same random inputs in every run."""

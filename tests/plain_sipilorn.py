@@ -162,8 +162,6 @@ def table_experts(m: dict, P: dict, h: torch.Tensor, tokens: list) -> torch.Tens
 
 
 def feed_forward(m, P: dict, h: torch.Tensor, tokens: list):
-    if m is None:
-        return torch.zeros_like(h)
     if m["kind"] == "dense":
         return dense_ff(P, h)
     if m["kind"] == "moe":
@@ -207,8 +205,9 @@ def forward(cfg: dict, P: dict, tokens: list, streams: list | None = None) -> to
             x = x + P["loop.step"][t]
         W = sub(P, f"l{i}.")
         a = mixer(L["type"], L["mixer"], sub(W, "mix."), rms_norm(x, W["norm1"], eps), eps)
-        f = feed_forward(L.get("mlp"), sub(W, "mlp."), rms_norm(x, W["norm2"], eps), tokens)
-        x = x + (a + f)
+        if L.get("mlp") is not None:
+            a = a + feed_forward(L["mlp"], sub(W, "mlp."), rms_norm(x, W["norm2"], eps), tokens)
+        x = x + a
         if streams is not None:
             streams.append(x.clone())
     z = rms_norm(x, P["final.norm"], eps) @ P["head"].T
