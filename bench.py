@@ -82,7 +82,36 @@ NETOVIK_SHAPES = {
                       dense_ff=12288, experts=32, top=4, expert_ff=1536)),
 }
 
-DESIGNS = {"disunex": ("Disunex", DISUNEX_SHAPES, disunex_shape), "netovik": ("Netovik", NETOVIK_SHAPES, netovik_shape)}
+def sipilorn_shape(width, delta_heads, delta_kv_heads, delta_dim, delta_vdim, heads, kv_heads, dim, window, pair_heads,
+                   dense_ff, experts, top, expert_ff, layers, vocab=151936):
+    """A Sipilorn configuration of ``layers`` layers: two layers of the gated delta rule, then one whose mixer is a
+    windowed attention beside a smaller recurrence, and so on; dense feed-forwards and experts by the table in turn."""
+    rec = {"type": "delta", "mixer": {"heads": delta_heads, "kv_heads": delta_kv_heads, "dim": delta_dim,
+                                      "vdim": delta_vdim, "conv": 4}}
+    par = {"type": "parallel", "mixer": {
+        "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                 "mask": {"size": window}, "rot": {"dims": dim // 2, "base": 1000000.0}},
+        "right": {"heads": pair_heads, "kv_heads": pair_heads, "dim": delta_dim, "vdim": delta_vdim, "conv": 4},
+        "left_scale": 1.0, "right_scale": 1.0}}
+    mlps = [{"kind": "dense", "ff": dense_ff},
+            {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}]
+    return {"architecture": "Sipilorn", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": [dict(par if i % 3 == 2 else rec, mlp=mlps[i % 2]) for i in range(layers)]}
+
+
+# Sipilorn at sizes that resemble a real model's layers, beside the Qwen3 shape of the same width (the same gated
+# feed-forward; the recurrence's q, k, v, gate and output are about four square matrices) and, with
+# --design-beside netovik, beside the design whose layers are closest: recurrences with a state per head and a
+# windowed attention every third layer
+SIPILORN_SHAPES = {
+    "2k": ("1.7b", dict(width=2048, delta_heads=16, delta_kv_heads=8, delta_dim=128, delta_vdim=128, heads=16, kv_heads=4,
+                        dim=128, window=1024, pair_heads=4, dense_ff=6144, experts=16, top=2, expert_ff=2048)),
+    "4k": ("8b", dict(width=4096, delta_heads=32, delta_kv_heads=16, delta_dim=128, delta_vdim=128, heads=32, kv_heads=8,
+                      dim=128, window=1024, pair_heads=8, dense_ff=12288, experts=32, top=4, expert_ff=3072)),
+}
+
+DESIGNS = {"disunex": ("Disunex", DISUNEX_SHAPES, disunex_shape), "netovik": ("Netovik", NETOVIK_SHAPES, netovik_shape),
+           "sipilorn": ("Sipilorn", SIPILORN_SHAPES, sipilorn_shape)}
 
 
 def design_points(args):
@@ -105,8 +134,12 @@ def design_points(args):
     for name in which:
         beside, sizes = shapes[name]
         row = {}
-        for label, cfg in ((args.design, make_shape(layers=L, **sizes)),
-                           ("qwen3_" + beside, dict(SHAPES[beside][1], num_hidden_layers=L))):
+        points = [(args.design, make_shape(layers=L, **sizes)),
+                  ("qwen3_" + beside, dict(SHAPES[beside][1], num_hidden_layers=L))]
+        if args.design_beside:      # a third column: another design at its own shape of this width
+            _, other_shapes, other_make = DESIGNS[args.design_beside]
+            points.append((args.design_beside, other_make(layers=L, **other_shapes[name][1])))
+        for label, cfg in points:
             if args.design_only and label != args.design_only and not label.startswith(args.design_only):
                 continue
             model = build_model(dict(cfg), args.seed)
@@ -179,6 +212,8 @@ def parse_args():
                          "throughput of this design at sizes that resemble a real model's layers, each beside the "
                          "Qwen3 shape of the same width, --layers layers each (default 8)")
     ap.add_argument("--design-shape", default=None, help="with --design: one of its sizes only (2k, 4k)")
+    ap.add_argument("--design-beside", choices=sorted(DESIGNS), default=None,
+                    help="with --design: also this other design at its own shape of the same width")
     ap.add_argument("--design-only", default=None, help="with --design: the design itself or 'qwen3' only (for profiling)")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "

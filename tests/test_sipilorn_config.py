@@ -208,3 +208,23 @@ def test_the_test_configurations_differ_from_each_other():
         seen.add(key)
     assert {L["type"] for L in SP_D["layers"]} == {"delta"} and "loop" not in SP_B and "logit_softcap" not in SP_C
     assert os.path.basename(__file__).startswith("test_")
+
+
+@pytest.mark.parametrize("name,layer", [("spA", 0), ("spB", 1)])
+def test_the_sharpened_weights_show_a_window_that_is_one_token_off_and_a_lost_state(tmp_path, name, layer):
+    """What the comparisons on the GPU rest on: in the plain implementation itself, a window one token longer or
+    shorter, or a request that goes on from an empty state, moves some row of logits by more than three tenths of
+    its largest entry, beyond what any row may differ by in the runs in bfloat16."""
+    from helpers import random_tokens, rel_err, tol
+    cfg, seed = SIPILORN_CONFIGS[name]
+    d = make_sipilorn_dir(str(tmp_path / name), cfg, seed)
+    c, P = plain.load(d)
+    toks = random_tokens(90, c["vocab"], 5)
+    ref = plain.forward(c, P, toks)
+    for dw in (-1, 1):
+        off = copy.deepcopy(c)
+        off["layers"][layer]["mixer"]["left"]["mask"]["size"] += dw
+        out = plain.forward(off, P, toks)
+        assert max(rel_err(out[i], ref[i]) for i in range(len(toks))) > 0.3 > 4 * tol("bfloat16", name)
+    tail = plain.forward(c, P, toks[50:])
+    assert max(rel_err(tail[i], ref[50 + i]) for i in range(len(tail))) > 0.3

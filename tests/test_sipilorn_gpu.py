@@ -1,0 +1,640 @@
+"""The Sipilorn design in the engine against the plain implementation: each mechanism alone at
+the level of its op or part, then whole models through the step function (whole prompts, decoding
+token by token, portions down to two tokens, mixed batches on a pool whose pages and slots are
+used again), and greedy generation through the engine's own entry point and scheduler."""
+import math
+import types
+
+import pytest
+import torch
+
+import plain_sipilorn as plain
+import replay_lib as rl
+from helpers import note_error, oracle_logits, random_tokens, read_config, rel_err, tol
+from sipilorn_models import SIPILORN_LENGTHS, SIPILORN_PAGE
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+NAMES = ["spA", "spB", "spC", "spD"]
+#: bfloat16: the share of a run's rows that may be over the tolerance, up to four times (rows at which the plain
+#: result's terms nearly cancel: an early token whose recurrence read-out is all but at right angles to its key,
+#: and the norm over the head then brings rounding up); the same rows in every way of cutting.  A window that is
+#: one token off or a lost state moves rows of these models by 0.7 of the largest logit and more.
+FEW = {"float32": 0.0, "bfloat16": 0.05}
+
+
+def _ops():
+    from tffinfer_amd.kernels import ops
+    return ops
+
+
+def _err(got, ref):
+    got, ref = _ops().as_tensor(got).double().cpu(), ref.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def _i32(v):
+    return torch.tensor(v, dtype=torch.int32, device=DEV)
+
+
+def _batch(lengths, starts, slots=None):
+    """The device tables of a step in which request r brings lengths[r] tokens after starts[r]."""
+    cu, pos, req = [0], [], []
+    for r, (n, s) in enumerate(zip(lengths, starts)):
+        cu.append(cu[-1] + n)
+        pos += list(range(s, s + n))
+        req += [r] * n
+    return types.SimpleNamespace(token_req=_i32(req), positions=_i32(pos), cu_tokens=_i32(cu), num_reqs=len(lengths),
+                                 num_tokens=cu[-1], max_new_tokens=max(lengths), host_cu_tokens=cu,
+                                 state_slots=_i32(slots if slots is not None else list(range(len(lengths)))))
+
+
+# ---------------------------------------------------------------- mechanisms, one by one ---
+
+@pytest.mark.parametrize("W", [48, 321, 1024, 5000])
+def test_two_norms_of_one_sum(W):
+    """resid += terms + a row; two RMS norms of the sum, each with a weight of its own; or the norms of chosen
+    rows with the stream left as it is."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(W)
+    n, eps = 6, 1e-3
+    x = torch.randn(n, W, generator=g) * 2
+    w1, w2 = (1 + 0.3 * torch.randn(W, generator=g) for _ in range(2))
+    bias = torch.randn(W, generator=g)
+    a = torch.randn(3, n, W, generator=g)
+    b = torch.randn(n, W, generator=g)
+    for terms, row, second in ((None, None, True), ([b], None, True), ([a, b], bias, True), ([a], bias, False),
+                               (None, bias, True)):
+        total = x.double() + (bias.double() if row is not None else 0)
+        for t in terms or []:
+            total = total + (t.double().sum(0) if t.dim() == 3 else t.double())
+        resid = x.clone().to(DEV)
+        delta = None if terms is None else (terms[0].to(DEV) if len(terms) == 1 else ops.PendingTerms([t.to(DEV) for t in terms]))
+        o1, o2 = ops.add_rmsnorm_pair(resid, delta, None if row is None else row.to(DEV), w1.to(DEV),
+                                      w2.to(DEV) if second else None, eps, torch.float32)
+        assert _err(resid, total) < 2e-6
+        assert _err(o1, plain.rms_norm(total, w1.double(), eps)) < 2e-6
+        assert (o2 is None) == (not second)
+        if second:
+            assert _err(o2, plain.rms_norm(total, w2.double(), eps)) < 2e-6
+    # chosen rows (the model's last norm), through the entry that norms of one weight use
+    resid = x.clone().to(DEV)
+    y = ops.add_rmsnorm(resid, ops.PendingTerms([a.to(DEV), b.to(DEV)]), w1.to(DEV), eps, torch.float32, rows=_i32([4, 0, 2]))
+    total = x.double() + a.double().sum(0) + b.double()
+    assert _err(y, plain.rms_norm(total, w1.double(), eps)[[4, 0, 2]]) < 2e-6
+    assert torch.equal(resid.cpu(), x)
+    # bfloat16 results are the float32 ones, rounded once
+    resid = x.clone().to(DEV)
+    h1, _ = ops.add_rmsnorm_pair(resid, b.to(DEV), None, w1.to(DEV), w2.to(DEV), eps, torch.bfloat16)
+    assert _err(h1.float(), plain.rms_norm(x.double() + b.double(), w1.double(), eps)) < 5e-3
+
+
+def test_the_cap_on_the_logits():
+    ops = _ops()
+    z = torch.linspace(-90, 90, 4001)
+    for cap in (5.0, 30.0):
+        got = ops.softcap_(z.clone().to(DEV), cap)
+        assert _err(got, cap * torch.tanh(z.double() / cap)) < 1e-6
+        assert float(got.abs().max()) <= cap
+
+
+@pytest.mark.parametrize("E,top", [(8, 3), (2, 2), (5, 1), (40, 4)])
+def test_experts_by_a_table_of_token_ids(E, top):
+    """No router: a row of the table per token id names the experts; each counts 1 / top; an expert is
+    down(relu(up x)^2), without a gate."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(E)
+    T, W, ff, V = 40, 48, 24, 70
+    x = torch.randn(T, W, generator=g)
+    table = torch.rand(V, E, generator=g).argsort(1)[:, :top].contiguous()
+    toks = torch.randint(0, V, (T,), generator=g)
+    toks[0], toks[1] = V - 1, 0
+    P = {"table": table}
+    for e in range(E):
+        P[f"e{e}.up"] = 0.3 * torch.randn(ff, W, generator=g).double()
+        P[f"e{e}.down"] = 0.3 * torch.randn(W, ff, generator=g).double()
+    ref = plain.table_experts({"router": {"top": top}}, P, x.double(), toks.tolist())
+    idx, wts = ops.route_by_table(table.to(torch.int32).to(DEV), toks.to(torch.int32).to(DEV), E)
+    assert torch.equal(idx.cpu().long(), table[toks]) and torch.equal(wts.cpu(), torch.full((T, top), 1.0 / top))
+    stack = lambda n: ops.pad_expert_rows(torch.stack([P[f"e{e}.{n}"] for e in range(E)], 0).float()).to(DEV)   # noqa: E731
+    out = ops.routed_experts(x.to(DEV), None, stack("up"), stack("down"), idx, wts, float("inf"), 1.0, up_offset=0.0)
+    assert _err(out, ref) < 2e-5
+    b16 = lambda t: t.to(torch.bfloat16)        # noqa: E731
+    for by_tiles in (False, True):
+        out = ops.routed_experts(b16(x).to(DEV), None, b16(stack("up")), b16(stack("down")), idx, wts,
+                                 float("inf"), 1.0, by_tiles=by_tiles, up_offset=0.0)
+        assert _err(out, ref) < 3e-2
+
+
+def _delta_case(T, H, G, D, E, taps, seed):
+    g = torch.Generator().manual_seed(seed)
+    C = 2 * G * D + H * E
+    proj = torch.randn(T, C + 2 * H + 5, generator=g) * 2          # (columns past b and a are someone else's)
+    proj[:, C + H:C + 2 * H] = 3 * torch.randn(T, H, generator=g) - 2      # decays from almost 0 to almost 1
+    conv = torch.randn(C, taps, generator=g) * 0.6
+    a_log = torch.rand(H, generator=g) * 3.5 - 3
+    dt = torch.randn(H, generator=g) * 0.5
+    return proj, conv, a_log, dt
+
+
+def _plain_delta(proj, conv, a_log, dt, H, G, D, E):
+    """o [T, H E] and nothing else, from the mechanism's plain functions."""
+    T = proj.shape[0]
+    p, cw = proj.double(), conv.double()
+    nq = G * D
+    q = plain.causal_conv_silu(p[:, :nq], cw[:nq]).view(T, G, D)
+    k = plain.causal_conv_silu(p[:, nq:2 * nq], cw[nq:2 * nq]).view(T, G, D)
+    v = plain.causal_conv_silu(p[:, 2 * nq:2 * nq + H * E], cw[2 * nq:]).view(T, H, E)
+    q = (plain.unit_vectors(q) * D ** -0.5).repeat_interleave(H // G, 1)
+    k = plain.unit_vectors(k).repeat_interleave(H // G, 1)
+    C = 2 * nq + H * E
+    beta = plain.sigmoid(p[:, C:C + H])
+    decay = torch.exp(-torch.exp(a_log.double()) * plain.softplus(p[:, C + H:C + 2 * H] + dt.double()))
+    return plain.delta_rule(q, k, v, beta, decay).reshape(T, H * E)
+
+
+@pytest.mark.parametrize("H,G,D,E,taps", [(3, 3, 8, 8, 4), (4, 2, 16, 24, 3), (2, 1, 24, 40, 2), (1, 1, 40, 16, 1),
+                                          (6, 2, 64, 17, 4), (2, 2, 100, 33, 5), (4, 1, 128, 64, 4), (1, 1, 192, 8, 2),
+                                          (2, 1, 256, 128, 4)])
+def test_delta_rule_whole_and_in_portions(H, G, D, E, taps):
+    """The recurrence over 70 tokens at once against the plain loop, and the same tokens in portions of 1 to 29
+    beside another request, with matrices and the convolution's last inputs carried in a slot: bit for bit
+    what the whole gave.  Slots that no request of a step names stay as they were."""
+    ops = _ops()
+    T = 70
+    proj, conv, a_log, dt = _delta_case(T, H, G, D, E, taps, D + E)
+    ref = _plain_delta(proj, conv, a_log, dt, H, G, D, E)
+    C = 2 * G * D + H * E
+    row = H * E * D + (taps - 1) * C
+    state = torch.zeros(4, row + 3, device=DEV)
+    dev = [t.to(DEV) for t in (conv, a_log, dt)]
+    whole = ops.gated_delta(proj.to(DEV), *dev, state, _batch([T], [0], [1]), H, G, D, E)
+    assert _err(whole, ref) < 3e-5
+    tail = state[1, H * E * D:row].view(taps - 1, C).cpu()
+    assert torch.equal(tail, proj[T - (taps - 1):, :C]) if taps > 1 else tail.numel() == 0
+    assert float(state[0].abs().max()) == 0 and float(state[2].abs().max()) == 0 and float(state[1, row:].abs().max()) == 0
+    final = state[1].clone()
+    # in portions, in slot 3, beside a second request in slot 0 whose tokens are some of the same ones
+    state.zero_()
+    got, at = [], 0
+    for n in (1, 2, 29, 1, 1, 7, 2, 27):
+        other = min(at + 1, T - n)
+        idx = list(range(at, at + n)) + [other]
+        o = ops.gated_delta(proj[idx].contiguous().to(DEV), *dev, state, _batch([n, 1], [at, 0], [3, 0]), H, G, D, E)
+        got.append(o[:n])
+        at += n
+    assert at == T
+    assert torch.equal(torch.cat(got, 0), whole)
+    assert torch.equal(state[3], final)
+    assert float(state[1].abs().max()) == 0 and float(state[2].abs().max()) == 0
+
+
+@pytest.mark.parametrize("decode", [False, True])
+def test_a_value_written_far_back_is_read(decode):
+    """Decay 1, beta 1, keys that are axes: the value written under an axis at the third token is what a query
+    along that axis reads 400 tokens later, whatever was written under the other axes since; with the axis
+    written once more in between, the later value.  As one prompt, and with the last 300 tokens decoded alone."""
+    ops = _ops()
+    H = G = 1
+    D, E, T = 16, 8, 403
+    C = 2 * D + E
+    g = torch.Generator().manual_seed(1)
+    proj = torch.full((T, C + 2), -30.0)
+    axis = [1 + (t % (D - 1)) for t in range(T)]
+    axis[2] = 0
+    for t in range(T):
+        proj[t, D + axis[t]] = 12.0                   # the key: an axis after silu and the unit norm
+        proj[t, 1 + (t % (D - 1))] = 12.0             # queries along the other axes
+    proj[T - 1, :D] = -30.0
+    proj[T - 1, 0] = 12.0                             # the last query: along the third token's key
+    proj[:, 2 * D:C] = torch.randn(T, E, generator=g) * 3
+    proj[:, C] = 30.0                                 # beta = 1
+    proj[:, C + 1] = -40.0                            # softplus = 0: no decay
+    conv = torch.ones(C, 1)
+    a_log, dt = torch.zeros(1), torch.zeros(1)
+    state = torch.zeros(2, E * D, device=DEV)
+    cuts = [103] + [1] * 300 if decode else [T]
+    outs, at = [], 0
+    for n in cuts:
+        outs.append(ops.gated_delta(proj[at:at + n].contiguous().to(DEV), conv.to(DEV), a_log.to(DEV), dt.to(DEV), state,
+                                    _batch([n], [at], [1]), H, G, D, E))
+        at += n
+    out = torch.cat(outs, 0).cpu()
+    v2 = plain.silu(proj[2, 2 * D:C].double())
+    assert torch.allclose(out[-1].double(), v2 * D ** -0.5, atol=1e-5)
+    assert _err(out, _plain_delta(proj, conv, a_log, dt, H, G, D, E)) < 1e-5
+    # the axis written once more at token 200: the last query reads that value
+    proj[200, D:2 * D] = -30.0
+    proj[200, D] = 12.0
+    state.zero_()
+    out = ops.gated_delta(proj.to(DEV), conv.to(DEV), a_log.to(DEV), dt.to(DEV), state, _batch([T], [0], [0]), H, G, D, E).cpu()
+    assert torch.allclose(out[-1].double(), plain.silu(proj[200, 2 * D:C].double()) * D ** -0.5, atol=1e-5)
+
+
+def test_the_convolution_starts_from_zeros_and_goes_on_from_the_state():
+    """A request's first tokens see zeros before them (not what the slot's last user left: the manager clears a
+    slot it hands out); a portion's first tokens see the portion before."""
+    ops = _ops()
+    H, G, D, E, taps, T = 2, 1, 8, 8, 4, 9
+    proj, conv, a_log, dt = _delta_case(T, H, G, D, E, taps, 11)
+    ref = _plain_delta(proj, conv, a_log, dt, H, G, D, E)
+    C = 2 * G * D + H * E
+    state = torch.zeros(1, H * E * D + (taps - 1) * C, device=DEV)
+    dev = [t.to(DEV) for t in (conv, a_log, dt)]
+    for cuts in ([1] * T, [2, 1, 2, 4], [T]):
+        state.zero_()
+        outs, at = [], 0
+        for n in cuts:
+            outs.append(ops.gated_delta(proj[at:at + n].contiguous().to(DEV), *dev, state, _batch([n], [at], [0]), H, G, D, E))
+            at += n
+        assert _err(torch.cat(outs, 0), ref) < 2e-5, cuts
+    # a slot that is not cleared gives something else: the test would see a manager that forgets to
+    stale = ops.gated_delta(proj.to(DEV), *dev, state, _batch([T], [0], [0]), H, G, D, E)
+    assert _err(stale, ref) > 1e-2
+
+
+@pytest.mark.parametrize("H,E", [(3, 8), (2, 40), (1, 128), (5, 17)])
+def test_norm_over_each_head_and_gates(H, E):
+    ops = _ops()
+    g = torch.Generator().manual_seed(H)
+    T, eps = 9, 1e-4
+    o, gz = 5 * torch.randn(T, H * E, generator=g), 2 * torch.randn(T, H * E + 6, generator=g)
+    w = 1 + 0.3 * torch.randn(E, generator=g)
+    ref = (plain.unit_rms(o.double().view(T, H, E), eps) * w.double()).reshape(T, H * E) * plain.silu(gz[:, 6:].double())
+    wide = torch.zeros(T, H * E + 10, device=DEV)
+    got = ops.head_norm_silu_gate(o.to(DEV), gz.to(DEV)[:, 6:], w.to(DEV), eps, H, E, wide[:, 10:], 0.7)
+    assert _err(got, 0.7 * ref) < 2e-6 and float(wide[:, :10].abs().max()) == 0
+    # the attention's gate: the first E elements of heads that lie P apart, times a sigmoid
+    P = E + 5
+    a = torch.randn(T, H * P, generator=g)
+    ref = (a.double().view(T, H, P)[:, :, :E].reshape(T, H * E)) * plain.sigmoid(gz[:, :H * E].double())
+    wide.zero_()
+    got = ops.sigmoid_gate_heads(a.to(DEV), P, gz.to(DEV)[:, :H * E], H, E, wide[:, :H * E], 1.3)
+    assert _err(got, 1.3 * ref) < 2e-6 and float(wide[:, H * E:].abs().max()) == 0
+
+
+def _ctx(cache, entries, act_dtype, max_positions=1024, cache_id=0):
+    from tffinfer_amd.engine.batch import KVView, build_step_batch
+    from tffinfer_amd.engine.runner import LayerContext
+    for e in entries:
+        if not cache.has_request(e.req):
+            cache.add_request(e.req)
+        cache.reserve(e.req, len(e.tokens))
+    batch = build_step_batch(entries, cache, DEV)
+    ctx = LayerContext(_ops(), act_dtype, batch, max_positions)
+    gi = cache.group_index(cache_id)
+    k, v = cache.kv_tensors(cache_id)
+    gt = batch.groups[gi]
+    ctx.kv = KVView(k, v, gt.block_tables, gt.slot_mapping, cache.page_size, gi)
+    return ctx
+
+
+def _attention_part(W, H, G, D, E, scale, window, rot, eps, dtype, seed, weights=None):
+    from tffinfer_amd.config.base import PartSpec
+    from tffinfer_amd.parts import GatedGQAttention
+    pos = PartSpec("rope", {"head_dim": D, "theta": rot[1], "pairing": "half", "rotary_dim": rot[0]}) if rot else None
+    att = GatedGQAttention(hidden_size=W, num_heads=H, num_kv_heads=G, head_dim=D, value_dim=E, position=pos, scale=scale,
+                           qk_norm_eps=eps, window=window)
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for k, s in att.weight_specs().items():
+        t = torch.randn(s.shape, generator=g)
+        w[k] = (1 + 0.2 * t) if s.init == "norm" else (t * 0.3).to(torch.bfloat16)
+    w.update(weights or {})
+    att.load_weights(w, dtype, DEV)
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": E, "scale": scale}
+    if window:
+        m["mask"] = {"size": window}
+    if rot:
+        m["rot"] = {"dims": rot[0], "base": rot[1]}
+    return att, m, {k: v.double() for k, v in w.items()}
+
+
+def _run_part(att, x, cuts, dtype, page, inner=False):
+    """The part over rows x of one request in portions ``cuts``; pages of a window go back as it moves on."""
+    from tffinfer_amd.cache import CacheManager
+    from tffinfer_amd.engine.batch import StepEntry
+    T = x.shape[0]
+    pages = -(-T // page) + 2
+    cache = CacheManager([(0, True, att.cache_spec(), None)], page, pages, 2, dtype=dtype, device=DEV)
+    outs, at = [], 0
+    for n in cuts:
+        ctx = _ctx(cache, [StepEntry("r", [0] * n, [])], dtype)
+        rows = x[at:at + n].to(dtype).to(DEV)
+        outs.append(_ops().as_tensor(att.forward_inner(ctx, rows) if inner else att.forward(ctx, rows)).float())
+        cache.commit("r", n)
+        at += n
+    assert at == T
+    return torch.cat(outs, 0)
+
+
+@pytest.mark.parametrize("dtype,limit", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("H,G,D,E,window,rot,page", [
+    (4, 2, 16, 24, 13, (8, 10000.0), 16),       # values wider than keys, a part of the head rotated
+    (6, 2, 32, 16, 0, None, 8),                 # narrower, no window, no rotation
+    (3, 3, 24, 40, 70, (24, 1e6), 32),          # the whole head rotated, a window over several pages
+    (2, 1, 64, 64, 8, (64, 500.0), 8),          # a window of one page
+    (5, 1, 40, 8, 33, (20, 50.0), 16),
+    (8, 2, 128, 128, 50, (64, 1e4), 16)])
+def test_gated_window_attention_part(H, G, D, E, window, rot, page, dtype, limit):
+    """Query and key norm with one weight for all heads, rotation in halves of the rotated part, the window, keys and
+    values of sizes of their own, the sigmoid gate, the output matrix: a prompt in one step, as portions down
+    to two tokens, and as a portion followed by single tokens, past the window."""
+    W, T, eps, scale = 48, 150, 1e-5, 0.25
+    att, m, P = _attention_part(W, H, G, D, E, scale, window, rot, eps, dtype, H * D + E)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(T, W, generator=g).to(torch.bfloat16).float()
+    ref = plain.window_attention(m, P, x.double(), eps)
+    for cuts in ([T], [3, 2, 61, 64, 20], [90] + [1] * 60):
+        err = _err(_run_part(att, x, cuts, dtype, page), ref)
+        assert err < limit, f"cut {cuts[:3]}: {err:.3e}"
+
+
+@pytest.mark.parametrize("decode", [False, True])
+@pytest.mark.parametrize("edge", ["inside", "outside"])
+def test_a_loud_key_at_the_windows_edge(edge, decode):
+    """One key whose score with the last query stands far out among 300 (the others are at right angles to the
+    query): just inside the window the head's output is that key's value, just outside it is not.  Across
+    page borders, in a prompt and in decoding."""
+    W = D = 16
+    H, G, E, T, page, window, eps = 2, 1, 24, 300, 16, 130, 1e-6
+    j = T - window if edge == "inside" else T - window - 1
+    eye = torch.eye(D).to(torch.bfloat16)
+    turn = torch.roll(eye, 2, dims=1)              # queries are the rows' elements two places on: q[3] = x[5]
+    fixed = {"q": torch.cat([turn, turn], 0), "k": eye, "q.norm": torch.ones(D), "k.norm": torch.ones(D)}
+    att, m, P = _attention_part(W, H, G, D, E, 1.5, window, None, eps, torch.float32, 5, weights=fixed)
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(T, W, generator=g).to(torch.bfloat16).float()
+    x[:, 3] = 0                                    # every key at right angles to axis 3 ...
+    x[j] = 0
+    x[j, 3] = 3.0                                  # ... but token j's, which lies along it
+    x[T - 1] = 0
+    x[T - 1, 5] = 2.0                              # the last query lies along axis 3, its own key along axis 5
+    out = _run_part(att, x, [T - 1, 1] if decode else [T], torch.float32, page, inner=True)
+    value = (x[j].double() @ P["v"].T)[:E]                      # the one kv head's value of token j
+    gate = plain.sigmoid(x[T - 1].double() @ P["g"].T)[E:2 * E]
+    near = torch.allclose(out[-1, E:2 * E].double().cpu(), value * gate, atol=2e-2, rtol=2e-2)
+    assert near == (edge == "inside"), edge
+    ref = plain.window_attention(m, P, x.double(), eps)
+    assert _err(out @ P["o"].T.float().to(DEV), ref) < 3e-5
+
+
+def test_batches_of_unequal_requests_share_the_mixers():
+    """Three requests in one step (a prompt's portion, a single token, a whole short prompt) through the pair of
+    attention and recurrence give what each gives alone, to rounding; freed pages and slots are used again."""
+    from tffinfer_amd.cache import CacheManager
+    from tffinfer_amd.config.base import PartSpec
+    from tffinfer_amd.engine.batch import KVView, StepEntry, build_step_batch
+    from tffinfer_amd.engine.runner import LayerContext
+    from tffinfer_amd.parts import MixerPair
+    W, eps, page = 40, 1e-5, 8
+    left = PartSpec("gated_gqa_attention", dict(hidden_size=W, num_heads=4, num_kv_heads=2, head_dim=16, value_dim=8, scale=0.3,
+                                                qk_norm_eps=eps, window=21,
+                                                position=PartSpec("rope", {"head_dim": 16, "theta": 100.0, "pairing": "half",
+                                                                           "rotary_dim": 8})))
+    right = PartSpec("gated_delta", dict(hidden_size=W, num_heads=2, num_kv_heads=1, head_dim=24, value_dim=16, conv_taps=3,
+                                         norm_eps=eps))
+    pair = MixerPair(W, left, right, 0.8, 1.7)
+    g = torch.Generator().manual_seed(2)
+    w = {}
+    for k, s in pair.weight_specs().items():
+        t = torch.randn(s.shape, generator=g)
+        w[k] = (1 + 0.2 * t) if s.init == "norm" else (3.5 * torch.rand(s.shape, generator=g) - 3 if s.init == "decay_log"
+                                                       else (t * 0.5 if s.init == "vector" else (t * 0.3).to(torch.bfloat16)))
+    pair.load_weights(w, torch.float32, DEV)
+    P = {k: v.double() for k, v in w.items()}
+    m = {"left": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 8, "scale": 0.3, "mask": {"size": 21},
+                  "rot": {"dims": 8, "base": 100.0}},
+         "right": {"heads": 2, "kv_heads": 1, "dim": 24, "vdim": 16, "conv": 3}, "left_scale": 0.8, "right_scale": 1.7}
+    lengths = [60, 41, 7]
+    xs = [torch.randn(n, W, generator=g).to(torch.bfloat16).float() for n in lengths]
+    refs = [plain.mixer("parallel", m, P, x.double(), eps) for x in xs]
+    cache = CacheManager([(0, True, pair.cache_spec(), pair.state_spec())], page, 18, 3, dtype=torch.float32, device=DEV)
+
+    def step(parts):
+        entries = [StepEntry(f"r{r}", [0] * (hi - lo), []) for r, lo, hi in parts]
+        for e in entries:
+            if not cache.has_request(e.req):
+                cache.add_request(e.req)
+            cache.reserve(e.req, len(e.tokens))
+        batch = build_step_batch(entries, cache, DEV)
+        ctx = LayerContext(_ops(), torch.float32, batch, 256)
+        gt = batch.groups[cache.group_index(0)]
+        k, v = cache.kv_tensors(0)
+        ctx.kv = KVView(k, v, gt.block_tables, gt.slot_mapping, page, cache.group_index(0))
+        ctx.state = cache.state_tensors[0]
+        out = _ops().as_tensor(pair.forward(ctx, torch.cat([xs[r][lo:hi] for r, lo, hi in parts], 0).to(DEV)))
+        at = 0
+        for (r, lo, hi), e in zip(parts, entries):
+            assert _err(out[at:at + hi - lo], refs[r][lo:hi]) < 3e-5, (r, lo, hi)
+            at += hi - lo
+            cache.commit(e.req, hi - lo)
+
+    step([(0, 0, 35), (1, 0, 40)])
+    step([(0, 35, 60), (1, 40, 41), (2, 0, 7)])
+    for r in range(3):
+        cache.release(f"r{r}")
+    # the same slots and pages again, for other requests
+    xs[0], xs[1] = xs[1], xs[0]
+    refs[0], refs[1] = refs[1], refs[0]
+    step([(1, 0, 2), (0, 0, 30)])
+    step([(1, 2, 60), (0, 30, 41)])
+    cache.check()
+
+
+# ---------------------------------------------------------------------- whole models ---
+
+def requests_for(name, model_dir):
+    V = read_config(model_dir)["vocab"]
+    return {f"{name}{i}": random_tokens(n, V, 3000 + 13 * i + n) for i, n in enumerate(SIPILORN_LENGTHS[name])}
+
+
+def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=4, use_graphs=False):
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.models import load_model
+    model = load_model(model_dir, DTYPES[dtype], DEV)
+    return ModelRunner(model, page_size=page_size, num_pages=num_pages, max_seqs=max_seqs, max_model_len=512,
+                       use_graphs=use_graphs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+def test_residual_stream_after_every_layer(sipilorn_dirs, name, dtype):
+    """Layer by layer, so that a fault names its layer.  A block leaves its two outputs to the block after it;
+    the stream after a layer run is the stream plus what is pending."""
+    from tffinfer_amd.engine.batch import StepEntry, build_step_batch
+    from tffinfer_amd.engine.runner import StepContext
+    d = sipilorn_dirs[name]
+    toks = random_tokens(45, read_config(d)["vocab"], 77)
+    want = []
+    plain.forward(*plain.load(d), toks, want)
+    runner = make_runner(d, dtype, SIPILORN_PAGE[name], 16)
+    model, ops = runner.model, runner.ops
+    runner.add_request("a")
+    e = [StepEntry("a", toks, [])]
+    runner.reserve(e)
+    batch = build_step_batch(e, runner.cache, runner.device, runner._pinned)
+    ctx = StepContext(ops, runner.act_dtype, batch, runner.max_model_len, runner._calls, runner.cache)
+    resid, pending = model.embedding.forward(ctx, batch.token_ids), None
+    assert len(model.schedule) == len(want)
+    for it, call in enumerate(model.schedule):
+        c = ctx.for_call(it)
+        if call.offset >= 0:
+            c.stream_offset = model.stream_offsets.row(call.offset)
+        pending = model.blocks[call.layer].forward(c, resid, pending)
+        after = resid + ops.as_tensor(pending)
+        err = _err(after, want[it])
+        assert err < (4e-5 if dtype == "float32" else 1e-1), f"layer call {it} (layer {call.layer}): {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("mode", ["whole", "tail", "chunks", "mixed"])
+def test_replay_modes(sipilorn_dirs, name, dtype, mode):
+    model_dir = sipilorn_dirs[name]
+    reqs = requests_for(name, model_dir)
+    steps = {"whole": rl.trace_whole, "tail": rl.trace_tail, "chunks": rl.trace_chunks,
+             "mixed": rl.trace_mixed}[mode](reqs)
+    ps = SIPILORN_PAGE[name]
+    # the pool holds what is live at the worst moment and no more, so pages and slots are used again
+    num_pages = rl.max_live_tokens(steps, unit=ps) // ps
+    runner = make_runner(model_dir, dtype, ps, num_pages)
+    results = rl.run_steps_in_process(runner, steps)
+    worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype, few_over=FEW[dtype])
+    print(f"{name} {dtype} {mode}: worst rel. error {worst:.3e} over {len(steps)} steps, {num_pages} pages")
+    assert all(g.pool.num_used == 0 for g in runner.cache.groups)
+
+
+def test_a_windows_pages_go_back(sipilorn_dirs):
+    """While a request grows far past its window, the group with the window holds the window's pages and no more."""
+    from tffinfer_amd.engine.batch import StepEntry
+    d = sipilorn_dirs["spA"]
+    ps = SIPILORN_PAGE["spA"]
+    toks = random_tokens(150, read_config(d)["vocab"], 2150)
+    runner = make_runner(d, "float32", ps, 12)
+    runner.add_request("a")
+    ref = oracle_logits(d, toks)
+    at = 0
+    for n in [50] + [1] * 100:
+        lg = runner.step([StepEntry("a", toks[at:at + n], [n - 1])])
+        at += n
+        assert rel_err(lg[0], ref[at - 1]) <= tol("float32", "spA")
+    seen = 0
+    for g in runner.cache.groups:
+        if g.spec.window:
+            held = [b for b, p in enumerate(g.tables["a"]) if p >= 0]
+            assert len(held) <= -(-(g.spec.window - 1) // ps) + 1 and held[0] > 0
+            seen += 1
+    assert seen
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["spA", "spC"])
+def test_long_decoding_through_captured_graphs(sipilorn_dirs, name, dtype):
+    """Three requests decode some 150 tokens each, far past every window, as replays of captured
+    HIP graphs beside eager prompt steps; state slots and pages of windows are used again."""
+    model_dir = sipilorn_dirs[name]
+    V = read_config(model_dir)["vocab"]
+    reqs = {f"g{i}": random_tokens(n, V, 300 + n) for i, n in enumerate((160, 171, 190))}
+    steps = rl.trace_mixed(reqs, max_live=3, prompt_frac=0.1, want_all=True)
+    ps = SIPILORN_PAGE[name]
+    runner = make_runner(model_dir, dtype, ps, rl.max_live_tokens(steps, unit=ps) // ps, use_graphs=True)
+    results = rl.run_steps_in_process(runner, steps)
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype, few_over=FEW[dtype])
+    assert runner._graphs, "no decode step ran as a graph"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(sipilorn_dirs, tmp_path, dtype):
+    """The program itself, as a user calls it, on a model of this architecture, with its four state slots."""
+    model_dir = sipilorn_dirs["spB"]
+    reqs = requests_for("spB", model_dir)
+    steps = rl.trace_mixed(reqs, want_all=False)
+    out = rl.run_steps_subprocess(model_dir, dtype, steps, str(tmp_path / "out"), rl.max_live_tokens(steps, 64))
+    rl.check_against_oracle(model_dir, reqs, steps, out, tol(dtype, "spB"), dtype, few_over=FEW[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["spA", "spB"])
+def test_greedy_generation_through_the_engine(sipilorn_dirs, name, dtype):
+    """The engine's own entry point: scheduler, portions beside decoding requests, graphs, sampler.
+    Every kept row of logits matches the plain logits of the engine's own sequence, and every
+    token is the first maximum of its row."""
+    from tffinfer_amd import EngineOptions, LLMEngine
+    d = sipilorn_dirs[name]
+    V = read_config(d)["vocab"]
+    prompts = [random_tokens(n, V, 80 + n) for n in (1, 9, 40, 70)]
+    eng = LLMEngine.from_model_dir(d, EngineOptions(dtype=dtype, page_size=16, kv_tokens=512, max_num_seqs=3,
+                                                    max_num_batched_tokens=48, prefill_chunk=24, max_model_len=256))
+    eng.keep_logits = True
+    res = eng.generate(prompts, max_new_tokens=40, ignore_eos=True)
+    over = 0
+    for r in res:
+        assert len(r.output) == 40 and r.finish_reason == "length"
+        ref = oracle_logits(d, r.prompt + r.output)
+        for i, (row, tok) in enumerate(zip(r.logits, r.output)):
+            assert tok == int(torch.argmax(row))
+            err = rel_err(row, ref[len(r.prompt) + i - 1])
+            if FEW[dtype] and tol(dtype, d) < err <= 4 * tol(dtype, d):
+                over += 1
+                continue
+            note_error(dtype, d, err)
+            assert err <= tol(dtype, d), f"output {i}: {err:.3e}"
+    assert over <= max(1, int(FEW[dtype] * 160))
+    if dtype == "float32":
+        cfg, W = plain.load(d)
+        toks = list(prompts[1])
+        for _ in range(8):
+            toks.append(int(torch.argmax(plain.forward(cfg, W, toks)[-1])))
+        assert res[1].output[:8] == toks[len(prompts[1]):]
+
+
+def test_a_preempted_request_starts_its_state_again(sipilorn_dirs):
+    """A pool so small that requests are preempted and computed again gives the tokens of a large pool:
+    the state of a request that comes back starts at zero."""
+    from tffinfer_amd import EngineOptions, LLMEngine
+    d = sipilorn_dirs["spC"]        # (its first layer keeps every key, so a small pool runs out)
+    V = read_config(d)["vocab"]
+    prompts = [random_tokens(n, V, 400 + n) for n in (30, 33, 28)]
+    outs, preempted = [], []
+    for pages in (64, 9):
+        eng = LLMEngine.from_model_dir(d, EngineOptions(dtype="float32", page_size=16, num_pages=pages, max_num_seqs=3,
+                                                        max_model_len=128))
+        res = eng.generate(prompts, max_new_tokens=30, ignore_eos=True)
+        outs.append([r.output for r in res])
+        preempted.append(sum(r.num_preemptions for r in res))
+    assert outs[0] == outs[1]
+    assert preempted[0] == 0 and preempted[1] > 0
+
+
+def test_the_command_line_with_a_configuration_file_of_this_architecture(tmp_path):
+    """--config FILE --random-weights through bin/tffinfer: the weights are those of the folder that
+    --save-model writes, the dumped rows are the logits that chose each token."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from sipilorn_models import SP_C
+    prog = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "tffinfer")
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(SP_C))
+    folder, dump = str(tmp_path / "spC"), str(tmp_path / "logits.f32")
+    cmd = [sys.executable, prog, "--config", str(cfg), "--random-weights", "--seed", "5", "--fp32", "--n-ctx", "256",
+           "--n-predict", "12", "--ignore-eos", "--json", "--random-prompts", "3:30", "--page-size", "8",
+           "--max-batches", "3", "--save-model", folder, "--dump-logits", dump, "--kv-tokens", "512"]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-3000:]
+    recs = [json.loads(ln) for ln in p.stdout.strip().splitlines()]
+    meta = json.load(open(dump + ".json"))
+    V = SP_C["vocab"]
+    rows = np.fromfile(dump, dtype="<f4").reshape(meta["shape"])
+    assert meta["shape"] == [36, V]
+    for i, r in enumerate(recs):
+        ref = oracle_logits(folder, r["prompt"] + r["output"])
+        first = meta["requests"][i]["first_row"]
+        for j, tok in enumerate(r["output"]):
+            row = torch.from_numpy(rows[first + j].copy())
+            assert rel_err(row, ref[len(r["prompt"]) - 1 + j]) <= tol("float32", "spC")
+            assert tok == int(torch.argmax(row))

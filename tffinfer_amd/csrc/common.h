@@ -28,6 +28,19 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Sum over the sixteen lanes of a row (lanes 16 r .. 16 r + 15 of a wave), the result in all of them:
+// neighbours, pairs, the two quads of a half, the two halves (data-parallel primitives: no LDS); the order of
+// the additions is fixed.
+__device__ __forceinline__ float row16_sum(float v) {
+#define TFF_DPP(x, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xF, 0xF, true))
+    v += TFF_DPP(v, 0xB1);       // quad_perm [1, 0, 3, 2]
+    v += TFF_DPP(v, 0x4E);       // quad_perm [2, 3, 0, 1]
+    v += TFF_DPP(v, 0x141);      // row_half_mirror
+    v += TFF_DPP(v, 0x140);      // row_mirror
+#undef TFF_DPP
+    return v;
+}
+
 // Sum over a block of up to 1024 threads; `red` holds at least 17 floats.
 // Every thread gets the result.  The order of the additions is fixed.
 __device__ __forceinline__ float block_sum(float v, float* red) {

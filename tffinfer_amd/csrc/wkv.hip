@@ -275,18 +275,6 @@ __global__ __launch_bounds__(512) void wkv_recurrence_wave_kernel(
     }
 }
 
-// Sum over the sixteen lanes of a row, the result in all of them: neighbours, pairs, the two quads of a half,
-// the two halves (data-parallel primitives: no LDS); the order of the additions is fixed.
-__device__ __forceinline__ float row16_sum(float v) {
-#define WKV_DPP(x, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xF, 0xF, true))
-    v += WKV_DPP(v, 0xB1);       // quad_perm [1, 0, 3, 2]
-    v += WKV_DPP(v, 0x4E);       // quad_perm [2, 3, 0, 1]
-    v += WKV_DPP(v, 0x141);      // row_half_mirror
-    v += WKV_DPP(v, 0x140);      // row_mirror
-#undef WKV_DPP
-    return v;
-}
-
 // For long portions (prompts) of heads of 64 or 128 channels (D = 16 * KPT): a token's cost is what bounds a
 // prompt, since its tokens go one after the other.  Here a row of sixteen lanes shares a value channel, each
 // lane KPT key channels, so a token is KPT steps of four instructions and a sum over the row; a block of four
