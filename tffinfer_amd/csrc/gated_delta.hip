@@ -91,23 +91,14 @@ TFF_API int tff_gdelta_prep(const float* proj, size_t ldp, const float* wconv, i
     return tff_check_launch("gdelta_prep");
 }
 
-// Sum over the sixteen lanes that share a value channel (neighbours, pairs, quads, halves of the row), the
-// result in all of them; the order of the additions is fixed.
-__device__ __forceinline__ float gd_row16_sum(float v) {
-    v += __shfl_xor(v, 1, 64);
-    v += __shfl_xor(v, 2, 64);
-    v += __shfl_xor(v, 4, 64);
-    v += __shfl_xor(v, 8, 64);
-    return v;
-}
-
 // Block: sixteen value channels of one head of one request; a row of sixteen lanes shares a value channel, each
 // lane KPL key channels of it (dim <= 16 KPL; the channels past dim are zero).  The tokens of the portion pass in
-// chunks of sixteen (eight for the widest heads): a chunk's k, q, its sixteen v, beta and decay are fetched into registers while the chunk
-// before is worked through from LDS, so that no token waits for memory; the waves meet at the chunks' borders
-// only.  Per token a lane does 5 KPL multiply-adds and three sums over its row:
-//   a = S^T k, b = S^T q (both of the state before the token), c = k . q;
-//   u = beta (v - g a);   o = g b + c u;   S <- g S + k u.
+// chunks of sixteen (eight for the widest heads): a chunk's k, q, its sixteen v, beta and decay are fetched into
+// registers while the chunk before is worked through from LDS, so that no token waits for memory; the waves meet
+// at the chunks' borders only.  Per token a lane does 4 KPL multiply-adds and two sums over its row:
+//   a = S^T k (of the state before the token);   u = beta (v - g a);   S <- g S + k u;   o = S^T q.
+// Only S runs from token to token; the read-out hangs off it, so with the loop unrolled by four a token's
+// read-out, its store and the LDS reads of the tokens after it fill the waits of the next token's sum.
 template <int KPL>
 __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
     const float* __restrict__ pre, const float* __restrict__ proj, size_t ldp, float* __restrict__ state, size_t state_row,
@@ -115,8 +106,9 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
     float* __restrict__ o, int H, int G, int D, int E) {
     constexpr int DP = 16 * KPL;
     constexpr int GD_CHUNK = KPL >= 16 ? 8 : 16;           // (two chunks of the widest heads fill LDS otherwise)
-    constexpr int ROWW = 2 * DP + 18;                      // k, q, sixteen v, beta, decay of a token
+    constexpr int ROWW = 2 * DP + 20;                      // k, q, sixteen v, beta, decay of a token; rows of 16 bytes
     constexpr int NLD = (GD_CHUNK * ROWW + 255) / 256;
+    constexpr int VEC = KPL % 4 == 0 ? 4 : (KPL % 2 == 0 ? 2 : 1);
     __shared__ __attribute__((aligned(16))) float lds[2][GD_CHUNK * ROWW];
     const int h = blockIdx.y, r = blockIdx.z, j0 = blockIdx.x * 16;
     const int tid = threadIdx.x, s = tid & 15, j = j0 + (tid >> 4);
@@ -130,57 +122,86 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
 #pragma unroll
     for (int m = 0; m < KPL; ++m) S[m] = (j < E && s * KPL + m < D) ? sp[m] : 0.f;
 
+    // (every element has one load at an address chosen without branches, so that the loads of a chunk are all in
+    // flight together; what lies past the portion, dim or vdim reads the first element and is stored as zero)
     float regs[NLD];
+    unsigned live = 0;
     auto fetch = [&](int first) {
+        live = 0;
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
             const int e = x * 256 + tid;
             const int tk = e / ROWW, col = e - tk * ROWW;
-            float v = 0.f;
-            if (tk < GD_CHUNK && first + tk < n) {
-                const float* p = pre + (size_t)(t0 + first + tk) * ldq;
-                if (col < DP) { if (col < D) v = p[(size_t)(G + gk) * D + col]; }
-                else if (col < 2 * DP) { if (col - DP < D) v = p[(size_t)gk * D + col - DP]; }
-                else if (col < 2 * DP + 16) { if (j0 + col - 2 * DP < E) v = p[2 * (size_t)G * D + (size_t)h * E + j0 + col - 2 * DP]; }
-                else v = p[C + (col - 2 * DP - 16) * H + h];
-            }
-            regs[x] = v;
+            const int ck = col, cq = col - DP, cv = col - 2 * DP, cb = col - 2 * DP - 16;
+            const bool isk = col < DP, isq = !isk && col < 2 * DP, isv = cv >= 0 && cv < 16, isb = cb >= 0 && cb < 2;
+            const bool ok = tk < GD_CHUNK && first + tk < n &&
+                            ((isk && ck < D) || (isq && cq < D) || (isv && j0 + cv < E) || isb);
+            const size_t at = isk ? (size_t)(G + gk) * D + ck
+                            : isq ? (size_t)gk * D + cq
+                            : isv ? 2 * (size_t)G * D + (size_t)h * E + j0 + cv
+                                  : (size_t)C + (size_t)cb * H + h;
+            const size_t off = ok ? (size_t)(t0 + first + tk) * ldq + at : 0;
+            regs[x] = pre[off];
+            live |= ok ? 1u << x : 0u;
         }
     };
     auto stash = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
             const int e = x * 256 + tid;
-            if (e < GD_CHUNK * ROWW) lds[buf][e] = regs[x];
+            if (e < GD_CHUNK * ROWW) lds[buf][e] = (live >> x & 1u) ? regs[x] : 0.f;
+        }
+    };
+    // a lane's KPL channels of a row of LDS, in reads of sixteen bytes where KPL allows
+    auto take = [&](const float* p, float* dst) {
+        if constexpr (VEC == 4) {
+#pragma unroll
+            for (int m = 0; m < KPL; m += 4) {
+                const float4 x = *reinterpret_cast<const float4*>(p + m);
+                dst[m] = x.x; dst[m + 1] = x.y; dst[m + 2] = x.z; dst[m + 3] = x.w;
+            }
+        } else if constexpr (VEC == 2) {
+#pragma unroll
+            for (int m = 0; m < KPL; m += 2) {
+                const float2 x = *reinterpret_cast<const float2*>(p + m);
+                dst[m] = x.x; dst[m + 1] = x.y;
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < KPL; ++m) dst[m] = p[m];
         }
     };
     fetch(0);
     stash(0);
     __syncthreads();
     int buf = 0;
+    const bool writer = s == 0 && j < E;
     for (int first = 0; first < n; first += GD_CHUNK) {
         const bool more = first + GD_CHUNK < n;
         if (more) fetch(first + GD_CHUNK);
         const int cnt = min(GD_CHUNK, n - first);
+        float* orow = o + (size_t)(t0 + first) * H * E + (size_t)h * E + min(j, E - 1);
+#pragma unroll 4
         for (int tk = 0; tk < cnt; ++tk) {
             const float* L = lds[buf] + tk * ROWW;
-            float a = 0.f, b = 0.f, c = 0.f, kk[KPL];
+            float kk[KPL], qq[KPL];
+            take(L + s * KPL, kk);
+            take(L + DP + s * KPL, qq);
+            const float v = L[2 * DP + (tid >> 4)];
+            const float2 bg = *reinterpret_cast<const float2*>(L + 2 * DP + 16);
+            float a = 0.f;
+#pragma unroll
+            for (int m = 0; m < KPL; ++m) a = fmaf(S[m], kk[m], a);
+            a = row16_sum(a);
+            const float u = bg.x * (v - bg.y * a);
+            float b = 0.f;
 #pragma unroll
             for (int m = 0; m < KPL; ++m) {
-                kk[m] = L[s * KPL + m];
-                const float qq = L[DP + s * KPL + m];
-                a = fmaf(S[m], kk[m], a);
-                b = fmaf(S[m], qq, b);
-                c = fmaf(kk[m], qq, c);
+                S[m] = fmaf(kk[m], u, bg.y * S[m]);
+                b = fmaf(S[m], qq[m], b);
             }
-            a = gd_row16_sum(a);
-            b = gd_row16_sum(b);
-            c = gd_row16_sum(c);
-            const float v = L[2 * DP + (tid >> 4)], beta = L[2 * DP + 16], g = L[2 * DP + 17];
-            const float u = beta * (v - g * a);
-#pragma unroll
-            for (int m = 0; m < KPL; ++m) S[m] = fmaf(kk[m], u, g * S[m]);
-            if (s == 0 && j < E) o[(size_t)(t0 + first + tk) * H * E + (size_t)h * E + j] = fmaf(c, u, g * b);
+            b = row16_sum(b);
+            if (writer) orow[(size_t)tk * H * E] = b;
         }
         if (more) stash(buf ^ 1);
         __syncthreads();
