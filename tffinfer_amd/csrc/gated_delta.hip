@@ -23,6 +23,7 @@
 #include "tffinfer_kernels.h"
 
 #define GD_MAX_TAPS 8
+#define GD_FEW 4        // tokens a request up to which a step counts as decoding
 
 __device__ __forceinline__ float gd_silu(float z) { return z / (1.0f + expf(-z)); }
 
@@ -91,8 +92,88 @@ TFF_API int tff_gdelta_prep(const float* proj, size_t ldp, const float* wconv, i
     return tff_check_launch("gdelta_prep");
 }
 
+// The convolution's last taps - 1 inputs go into the state: by the block of a head's first value channels, the
+// head's value channels, and with the first head of a group its q and k.
+__device__ __forceinline__ void gd_keep_inputs(const float* __restrict__ proj, size_t ldp, float* __restrict__ tail, int taps,
+                                               int t0, int n, int h, int gk, int H, int G, int D, int E) {
+    if (taps <= 1) return;
+    const int C = 2 * G * D + H * E;
+    const int own = (h % (H / G) == 0) ? 2 * D : 0;
+    for (int x = threadIdx.x; x < E + own; x += blockDim.x) {
+        const int c = x < E ? 2 * G * D + h * E + x : (x - E < D ? gk * D + x - E : (G + gk) * D + x - E - D);
+        for (int i = 0; i < taps - 1; ++i) {            // ascending: what is read lies behind what was written
+            const int src = n - (taps - 1) + i;
+            tail[(size_t)i * C + c] = src >= 0 ? proj[(size_t)(t0 + src) * ldp + c] : tail[(size_t)(i + n) * C + c];
+        }
+    }
+}
+
+// One token of one value channel, on the row of sixteen lanes that shares the channel; lane s holds the key
+// channels s, s + 16, ... of S, k and q.  The same additions in the same order wherever it is used, so that a
+// sequence gives the same bits however it is cut into steps.
+template <int KPL>
+__device__ __forceinline__ float gd_token(float (&S)[KPL], const float (&kk)[KPL], const float (&qq)[KPL], float v, float beta,
+                                          float g) {
+    float a = 0.f;
+#pragma unroll
+    for (int m = 0; m < KPL; ++m) a = fmaf(S[m], kk[m], a);
+    a = row16_sum(a);
+    const float u = beta * (v - g * a);
+    float b = 0.f;
+#pragma unroll
+    for (int m = 0; m < KPL; ++m) {
+        S[m] = fmaf(kk[m], u, g * S[m]);
+        b = fmaf(S[m], qq[m], b);
+    }
+    return row16_sum(b);
+}
+
+// For steps in which every request brings a few tokens (decoding): no LDS and no barrier.  A row of sixteen lanes
+// shares a value channel as above, but lane s takes the key channels s, s + 16, ...: a load or store of the state
+// is sixteen neighbouring floats a row, and k and q come straight from the prepared rows.
+template <int KPL>
+__global__ __launch_bounds__(256) void gdelta_recurrence_few_kernel(
+    const float* __restrict__ pre, const float* __restrict__ proj, size_t ldp, float* __restrict__ state, size_t state_row,
+    size_t tail_off, int taps, const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ state_slots,
+    float* __restrict__ o, int H, int G, int D, int E) {
+    const int h = blockIdx.y, r = blockIdx.z, j0 = blockIdx.x * 16;
+    const int tid = threadIdx.x, s = tid & 15, j = j0 + (tid >> 4), jc = min(j, E - 1);
+    const int C = 2 * G * D + H * E;
+    const size_t ldq = (size_t)C + 2 * H;
+    const int gk = h / (H / G);
+    const int t0 = cu_tokens[r], n = cu_tokens[r + 1] - t0;
+    float* srow = state + (size_t)state_slots[r] * state_row;
+    float* sp = srow + ((size_t)h * E + jc) * D + s;
+    const bool row_live = j < E;
+    float S[KPL];
+#pragma unroll
+    for (int m = 0; m < KPL; ++m) S[m] = (row_live && s + 16 * m < D) ? sp[16 * m] : 0.f;
+    for (int t = 0; t < n; ++t) {
+        const float* p = pre + (size_t)(t0 + t) * ldq;
+        const float* pk = p + (size_t)(G + gk) * D + s;
+        const float* pq = p + (size_t)gk * D + s;
+        float kk[KPL], qq[KPL];
+#pragma unroll
+        for (int m = 0; m < KPL; ++m) {
+            const bool in = s + 16 * m < D;
+            kk[m] = in ? pk[16 * m] : 0.f;
+            qq[m] = in ? pq[16 * m] : 0.f;
+        }
+        const float v = p[2 * (size_t)G * D + (size_t)h * E + jc], beta = p[C + h], g = p[C + H + h];
+        const float b = gd_token<KPL>(S, kk, qq, v, beta, g);
+        if (s == 0 && row_live) o[(size_t)(t0 + t) * H * E + (size_t)h * E + j] = b;
+    }
+    if (row_live) {
+#pragma unroll
+        for (int m = 0; m < KPL; ++m)
+            if (s + 16 * m < D) sp[16 * m] = S[m];
+    }
+    if (blockIdx.x == 0) gd_keep_inputs(proj, ldp, srow + tail_off, taps, t0, n, h, gk, H, G, D, E);
+}
+
 // Block: sixteen value channels of one head of one request; a row of sixteen lanes shares a value channel, each
-// lane KPL key channels of it (dim <= 16 KPL; the channels past dim are zero).  The tokens of the portion pass in
+// lane the KPL key channels s, s + 16, ... of it (dim <= 16 KPL; the channels past dim are zero; in LDS a lane's
+// channels of k and of q lie side by side).  The tokens of the portion pass in
 // chunks of sixteen (eight for the widest heads): a chunk's k, q, its sixteen v, beta and decay are fetched into
 // registers while the chunk before is worked through from LDS, so that no token waits for memory; the waves meet
 // at the chunks' borders only.  Per token a lane does 4 KPL multiply-adds and two sums over its row:
@@ -118,9 +199,9 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
     const int t0 = cu_tokens[r], n = cu_tokens[r + 1] - t0;
     float* srow = state + (size_t)state_slots[r] * state_row;
     float S[KPL];
-    float* sp = srow + ((size_t)h * E + min(j, E - 1)) * D + s * KPL;
+    float* sp = srow + ((size_t)h * E + min(j, E - 1)) * D + s;
 #pragma unroll
-    for (int m = 0; m < KPL; ++m) S[m] = (j < E && s * KPL + m < D) ? sp[m] : 0.f;
+    for (int m = 0; m < KPL; ++m) S[m] = (j < E && s + 16 * m < D) ? sp[16 * m] : 0.f;
 
     // (every element has one load at an address chosen without branches, so that the loads of a chunk are all in
     // flight together; what lies past the portion, dim or vdim reads the first element and is stored as zero)
@@ -149,7 +230,10 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
             const int e = x * 256 + tid;
-            if (e < GD_CHUNK * ROWW) lds[buf][e] = (live >> x & 1u) ? regs[x] : 0.f;
+            const int tk = e / ROWW, col = e - tk * ROWW;
+            const int d = col < DP ? col : col - DP;                       // key channel d: lane d % 16, its place d / 16
+            const int at = col < 2 * DP ? col - d + (d & 15) * KPL + (d >> 4) : col;
+            if (e < GD_CHUNK * ROWW) lds[buf][tk * ROWW + at] = (live >> x & 1u) ? regs[x] : 0.f;
         }
     };
     // a lane's KPL channels of a row of LDS, in reads of sixteen bytes where KPL allows
@@ -189,18 +273,7 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
             take(L + DP + s * KPL, qq);
             const float v = L[2 * DP + (tid >> 4)];
             const float2 bg = *reinterpret_cast<const float2*>(L + 2 * DP + 16);
-            float a = 0.f;
-#pragma unroll
-            for (int m = 0; m < KPL; ++m) a = fmaf(S[m], kk[m], a);
-            a = row16_sum(a);
-            const float u = bg.x * (v - bg.y * a);
-            float b = 0.f;
-#pragma unroll
-            for (int m = 0; m < KPL; ++m) {
-                S[m] = fmaf(kk[m], u, bg.y * S[m]);
-                b = fmaf(S[m], qq[m], b);
-            }
-            b = row16_sum(b);
+            const float b = gd_token<KPL>(S, kk, qq, v, bg.x, bg.y);
             if (writer) orow[(size_t)tk * H * E] = b;
         }
         if (more) stash(buf ^ 1);
@@ -210,25 +283,14 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
     if (j < E) {
 #pragma unroll
         for (int m = 0; m < KPL; ++m)
-            if (s * KPL + m < D) sp[m] = S[m];
+            if (s + 16 * m < D) sp[16 * m] = S[m];
     }
-    // the convolution's last inputs: the head's value channels, and with the first head of a group its q and k
-    if (blockIdx.x == 0 && taps > 1) {
-        float* tail = srow + tail_off;
-        const int own = (h % (H / G) == 0) ? 2 * D : 0;
-        for (int x = tid; x < E + own; x += 256) {
-            const int c = x < E ? 2 * G * D + h * E + x : (x - E < D ? gk * D + x - E : (G + gk) * D + x - E - D);
-            for (int i = 0; i < taps - 1; ++i) {            // ascending: what is read lies behind what was written
-                const int src = n - (taps - 1) + i;
-                tail[(size_t)i * C + c] = src >= 0 ? proj[(size_t)(t0 + src) * ldp + c] : tail[(size_t)(i + n) * C + c];
-            }
-        }
-    }
+    if (blockIdx.x == 0) gd_keep_inputs(proj, ldp, srow + tail_off, taps, t0, n, h, gk, H, G, D, E);
 }
 
 TFF_API int tff_gdelta_recurrence(const float* pre, const float* proj, size_t ldp, float* state, size_t state_row,
                                   size_t tail_off, int taps, const int32_t* cu_tokens, const int32_t* state_slots, float* o,
-                                  int R, int H, int G, int D, int E, tff_stream_t stream) {
+                                  int R, int H, int G, int D, int E, int max_tokens, tff_stream_t stream) {
     TFF_REQUIRE(pre && proj && state && cu_tokens && state_slots && o, "gdelta_recurrence: null pointer");
     TFF_REQUIRE(R >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && E > 0 && taps >= 1 && taps <= GD_MAX_TAPS,
                 "gdelta_recurrence: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d taps=%d (dim up to 256, taps up to %d)", H, G, D,
@@ -240,9 +302,16 @@ TFF_API int tff_gdelta_recurrence(const float* pre, const float* proj, size_t ld
     if (R == 0) return 0;
     const dim3 grid((E + 15) / 16, H, R);
     hipStream_t s = (hipStream_t)stream;
+    // (a request's tokens go one after the other: up to GD_FEW of them need no staging through LDS)
 #define GD_LAUNCH(KPL)                                                                                                     \
-    gdelta_recurrence_kernel<KPL><<<grid, 256, 0, s>>>(pre, proj, ldp, state, state_row, tail_off, taps, cu_tokens, state_slots, \
-                                                       o, H, G, D, E)
+    do {                                                                                                                   \
+        if (max_tokens > 0 && max_tokens <= GD_FEW)                                                                        \
+            gdelta_recurrence_few_kernel<KPL><<<grid, 256, 0, s>>>(pre, proj, ldp, state, state_row, tail_off, taps,        \
+                                                                   cu_tokens, state_slots, o, H, G, D, E);                 \
+        else                                                                                                               \
+            gdelta_recurrence_kernel<KPL><<<grid, 256, 0, s>>>(pre, proj, ldp, state, state_row, tail_off, taps, cu_tokens, \
+                                                               state_slots, o, H, G, D, E);                                \
+    } while (0)
     if (D <= 16) GD_LAUNCH(1);
     else if (D <= 32) GD_LAUNCH(2);
     else if (D <= 64) GD_LAUNCH(4);

@@ -323,10 +323,11 @@ TFF_API int tff_gdelta_prep(const float* proj, size_t ldp, const float* wconv, i
                             int T, int H, int G, int D, int E, tff_stream_t stream);
 // Per request (cu_tokens, state_slots) and head h (keys and queries of head h / (H / G)), S^T [E, D] at the start of
 // the state row: S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  o float32 [T, H * E].  The
-// portion's last taps - 1 rows of proj's channels are left at tail_off of the state row.
+// portion's last taps - 1 rows of proj's channels are left at tail_off of the state row.  max_tokens: the most
+// tokens that a request brings in this step (0: unknown); it chooses between the form for decoding and for prompts.
 TFF_API int tff_gdelta_recurrence(const float* pre, const float* proj, size_t ldp, float* state, size_t state_row,
                                   size_t tail_off, int taps, const int32_t* cu_tokens, const int32_t* state_slots, float* o,
-                                  int R, int H, int G, int D, int E, tff_stream_t stream);
+                                  int R, int H, int G, int D, int E, int max_tokens, tff_stream_t stream);
 // out[t * out_row + h * E + e] = o[t, h, e] / sqrt(mean over e of o^2 + eps) * w[e] * silu(g[t * g_row + h * E + e]) * scale
 TFF_API int tff_head_norm_silu_gate(const float* o, const float* g, size_t g_row, const float* w, float eps, float scale,
                                     void* out, size_t out_row, int T, int H, int E, int out_dtype, tff_stream_t stream);

@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 31
+ABI_VERSION = 32
 
 
 class KernelLibraryError(RuntimeError):
@@ -62,7 +62,7 @@ _SIGNATURES = {
     "tff_head_norm_gate": [_P, _P, _Z, _P, _F, _P, _I, _I, _I, _I, _P],
     "tff_tanh": [_P, _P, _Z, _I, _P],
     "tff_gdelta_prep": [_P, _Z, _P, _I, _P, _P, _P, _Z, _Z, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "tff_gdelta_recurrence": [_P, _P, _Z, _P, _Z, _Z, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "tff_gdelta_recurrence": [_P, _P, _Z, _P, _Z, _Z, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "tff_head_norm_silu_gate": [_P, _P, _Z, _P, _F, _F, _P, _Z, _I, _I, _I, _I, _P],
     "tff_sigmoid_gate_heads": [_P, _Z, _I, _P, _Z, _F, _P, _Z, _I, _I, _I, _I, _P],
     "tff_add_rmsnorm_pair": [_P, _P, _I, _Z, _P, _I, _Z, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P],

@@ -1505,7 +1505,7 @@ def gated_delta(proj: torch.Tensor, conv_w: torch.Tensor, a_log: torch.Tensor, d
                                  batch.state_slots.data_ptr(), pre.data_ptr(), T, H, G, D, E, stream))
     _lib.check(L.tff_gdelta_recurrence(pre.data_ptr(), proj.data_ptr(), ldp, state.data_ptr(), row, tail, taps,
                                        batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), o.data_ptr(),
-                                       batch.num_reqs, H, G, D, E, stream))
+                                       batch.num_reqs, H, G, D, E, int(getattr(batch, "max_new_tokens", 0) or 0), stream))
     return o
 
 
