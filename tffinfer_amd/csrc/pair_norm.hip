@@ -10,8 +10,12 @@
 
 #define PN_MAX_W 15360
 
-template <typename TO>
-__global__ __launch_bounds__(256) void add_rmsnorm_pair_kernel(
+// NT threads a block: 256 where the rows fill the GPU, 1024 for the few rows of a decode step (four elements a
+// thread instead of sixteen, so that a row's loads are in flight together).  The sum of squares is formed by the
+// first 256 threads from LDS, element e by thread e mod 256 in the order of e, whatever NT is: a row's norm does
+// not depend on how many rows the step has.
+template <typename TO, int NT>
+__global__ __launch_bounds__(NT) void add_rmsnorm_pair_kernel(
     float* __restrict__ resid, const float* __restrict__ d0, int planes0, size_t plane0, const float* __restrict__ d1,
     int planes1, size_t plane1, const float* __restrict__ bias, const float* __restrict__ w1, const float* __restrict__ w2,
     float eps, TO* __restrict__ out1, TO* __restrict__ out2, const int32_t* __restrict__ rows, int W) {
@@ -20,19 +24,23 @@ __global__ __launch_bounds__(256) void add_rmsnorm_pair_kernel(
     const int i = blockIdx.x;
     const size_t row = rows ? (size_t)rows[i] : (size_t)i;
     float* x = resid + row * W;
-    float ss = 0.f;
-    for (int e = threadIdx.x; e < W; e += 256) {
+    for (int e = threadIdx.x; e < W; e += NT) {
         float v = x[e];
+#pragma unroll 4
         for (int p = 0; p < planes0; ++p) v += d0[p * plane0 + row * W + e];
+#pragma unroll 4
         for (int p = 0; p < planes1; ++p) v += d1[p * plane1 + row * W + e];
         if (bias) v += bias[e];
         if (!rows) x[e] = v;
         vrow[e] = v;
-        ss = fmaf(v, v, ss);
     }
+    __syncthreads();
+    float ss = 0.f;
+    if (threadIdx.x < 256)
+        for (int e = threadIdx.x; e < W; e += 256) ss = fmaf(vrow[e], vrow[e], ss);
     ss = block_sum(ss, red);
     const float rr = 1.0f / sqrtf(ss / (float)W + eps);
-    for (int e = threadIdx.x; e < W; e += 256) {
+    for (int e = threadIdx.x; e < W; e += NT) {
         const float v = vrow[e] * rr;
         out1[(size_t)i * W + e] = from_f32<TO>(v * w1[e]);
         if (w2) out2[(size_t)i * W + e] = from_f32<TO>(v * w2[e]);
@@ -48,14 +56,17 @@ TFF_API int tff_add_rmsnorm_pair(float* resid, const float* d0, int planes0, siz
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = (size_t)W * sizeof(float);
-    if (out_dtype == TFF_F32)
-        add_rmsnorm_pair_kernel<float><<<n, 256, lds, s>>>(resid, d0, planes0, plane0, d1, planes1, plane1, bias, w1, w2, eps,
-                                                          (float*)out1, (float*)out2, rows, W);
-    else if (out_dtype == TFF_BF16)
-        add_rmsnorm_pair_kernel<bf16_t><<<n, 256, lds, s>>>(resid, d0, planes0, plane0, d1, planes1, plane1, bias, w1, w2, eps,
-                                                           (bf16_t*)out1, (bf16_t*)out2, rows, W);
-    else
+#define PN_LAUNCH(TO, NT)                                                                                              \
+    add_rmsnorm_pair_kernel<TO, NT><<<n, NT, lds, s>>>(resid, d0, planes0, plane0, d1, planes1, plane1, bias, w1, w2, eps, \
+                                                      (TO*)out1, (TO*)out2, rows, W)
+    const bool few = n <= 128 && W > 1024;
+    if (out_dtype == TFF_F32) {
+        if (few) PN_LAUNCH(float, 1024); else PN_LAUNCH(float, 256);
+    } else if (out_dtype == TFF_BF16) {
+        if (few) PN_LAUNCH(bf16_t, 1024); else PN_LAUNCH(bf16_t, 256);
+    } else
         return tff_fail("add_rmsnorm_pair: unknown dtype %d", out_dtype);
+#undef PN_LAUNCH
     return tff_check_launch("add_rmsnorm_pair");
 }
 
