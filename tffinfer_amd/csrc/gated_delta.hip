@@ -197,6 +197,7 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
     const size_t ldq = (size_t)C + 2 * H;
     const int gk = h / (H / G);
     const int t0 = cu_tokens[r], n = cu_tokens[r + 1] - t0;
+    if (n <= 0) return;                                    // (the whole block: a request without tokens changes nothing)
     float* srow = state + (size_t)state_slots[r] * state_row;
     float S[KPL];
     float* sp = srow + ((size_t)h * E + min(j, E - 1)) * D + s;
@@ -204,37 +205,42 @@ __global__ __launch_bounds__(256) void gdelta_recurrence_kernel(
     for (int m = 0; m < KPL; ++m) S[m] = (j < E && s + 16 * m < D) ? sp[16 * m] : 0.f;
 
     // (every element has one load at an address chosen without branches, so that the loads of a chunk are all in
-    // flight together; what lies past the portion, dim or vdim reads the first element and is stored as zero)
+    // flight together; what lies past the portion, dim or vdim reads the row's first element and is stored as zero.
+    // Where an element comes from and where it goes in LDS does not change from chunk to chunk: found once.)
     float regs[NLD];
-    unsigned live = 0;
+    unsigned rel[NLD], live = 0, cols = 0;
+    int dst[NLD], tks[NLD];
+#pragma unroll
+    for (int x = 0; x < NLD; ++x) {
+        const int e = x * 256 + tid;
+        const int tk = e / ROWW, col = e - tk * ROWW;
+        const int ck = col, cq = col - DP, cv = col - 2 * DP, cb = col - 2 * DP - 16;
+        const bool isk = col < DP, isq = !isk && col < 2 * DP, isv = cv >= 0 && cv < 16, isb = cb >= 0 && cb < 2;
+        const bool ok = tk < GD_CHUNK && ((isk && ck < D) || (isq && cq < D) || (isv && j0 + cv < E) || isb);
+        const size_t at = isk ? (size_t)(G + gk) * D + ck
+                        : isq ? (size_t)gk * D + cq
+                        : isv ? 2 * (size_t)G * D + (size_t)h * E + j0 + cv
+                              : (size_t)C + (size_t)cb * H + h;
+        rel[x] = ok ? (unsigned)((size_t)tk * ldq + at) : 0u;
+        cols |= ok ? 1u << x : 0u;
+        tks[x] = tk;
+        const int d = col < DP ? col : col - DP;                           // key channel d: lane d % 16, its place d / 16
+        dst[x] = e < GD_CHUNK * ROWW ? tk * ROWW + (col < 2 * DP ? col - d + (d & 15) * KPL + (d >> 4) : col) : -1;
+    }
     auto fetch = [&](int first) {
+        const float* base = pre + (size_t)(t0 + first) * ldq;
         live = 0;
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
-            const int e = x * 256 + tid;
-            const int tk = e / ROWW, col = e - tk * ROWW;
-            const int ck = col, cq = col - DP, cv = col - 2 * DP, cb = col - 2 * DP - 16;
-            const bool isk = col < DP, isq = !isk && col < 2 * DP, isv = cv >= 0 && cv < 16, isb = cb >= 0 && cb < 2;
-            const bool ok = tk < GD_CHUNK && first + tk < n &&
-                            ((isk && ck < D) || (isq && cq < D) || (isv && j0 + cv < E) || isb);
-            const size_t at = isk ? (size_t)(G + gk) * D + ck
-                            : isq ? (size_t)gk * D + cq
-                            : isv ? 2 * (size_t)G * D + (size_t)h * E + j0 + cv
-                                  : (size_t)C + (size_t)cb * H + h;
-            const size_t off = ok ? (size_t)(t0 + first + tk) * ldq + at : 0;
-            regs[x] = pre[off];
+            const bool ok = (cols >> x & 1u) && first + tks[x] < n;
+            regs[x] = base[ok ? rel[x] : 0u];
             live |= ok ? 1u << x : 0u;
         }
     };
     auto stash = [&](int buf) {
 #pragma unroll
-        for (int x = 0; x < NLD; ++x) {
-            const int e = x * 256 + tid;
-            const int tk = e / ROWW, col = e - tk * ROWW;
-            const int d = col < DP ? col : col - DP;                       // key channel d: lane d % 16, its place d / 16
-            const int at = col < 2 * DP ? col - d + (d & 15) * KPL + (d >> 4) : col;
-            if (e < GD_CHUNK * ROWW) lds[buf][tk * ROWW + at] = (live >> x & 1u) ? regs[x] : 0.f;
-        }
+        for (int x = 0; x < NLD; ++x)
+            if (dst[x] >= 0) lds[buf][dst[x]] = (live >> x & 1u) ? regs[x] : 0.f;
     };
     // a lane's KPL channels of a row of LDS, in reads of sixteen bytes where KPL allows
     auto take = [&](const float* p, float* dst) {
@@ -299,6 +305,7 @@ TFF_API int tff_gdelta_recurrence(const float* pre, const float* proj, size_t ld
     TFF_REQUIRE(ldp >= C + 2 * (size_t)H && (size_t)H * E * D <= tail_off && tail_off + (size_t)(taps - 1) * C <= state_row,
                 "gdelta_recurrence: rows of %zu or state rows of %zu are too short", ldp, state_row);
     TFF_REQUIRE(H <= 65535 && R <= 65535, "gdelta_recurrence: too many heads or requests");
+    TFF_REQUIRE((C + 2 * (size_t)H) * 17 < ((size_t)1 << 31), "gdelta_recurrence: rows of %zu channels are too long", C);
     if (R == 0) return 0;
     const dim3 grid((E + 15) / 16, H, R);
     hipStream_t s = (hipStream_t)stream;
