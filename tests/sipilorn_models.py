@@ -1,11 +1,11 @@
 """Tiny Sipilorn configurations for the tests, and their model folders.
 
-Sizes differ from layer to layer and between the configurations: key sizes of 8 to 192 and value
-sizes of 8 to 64 that are no multiples of each other (values wider and narrower than keys), one to six
-heads, grouped and ungrouped kv heads, windows of 8 to 70 and an attention without a window,
-rotations of a part of the head and of the whole head, convolutions of one to five taps, one to
-three experts a token, a layer without a feed-forward, loops over a part of the layers, over all
-of them, three passes, and no loop at all, with and without a cap on the logits.  The random weights
+Sizes differ from layer to layer and between the configurations: key sizes of 4 to 192 and value
+sizes of 4 to 64 that are no multiples of each other (values wider and narrower than keys), widths and
+feed-forwards that are no multiples of 8, one to seven heads, grouped and ungrouped kv heads, windows of
+1 to 70 and an attention without a window, rotations of a part of the head and of the whole head,
+convolutions of one to five taps, one expert a token to all of them, a layer without a feed-forward, loops
+over a part of the layers, over all of them, three passes, one pass, and no loop at all, with and without a cap on the logits.  The random weights
 are made *sharp* after they are drawn so that a wrong window edge, a lost state or a wrong expert
 moves the logits by far more than bfloat16 rounding.
 """
@@ -80,10 +80,17 @@ SP_D = model(48, 90, 1e-6, [
     layer("delta", delta(6, 3, 8, 8, 4), dense(56)),
     layer("delta", delta(2, 1, 128, 32, 3), moe(4, 1, 8)),
 ], loop=(0, 1, 2), softcap=8.0)
-SIPILORN_CONFIGS = {"spA": (SP_A, 3), "spB": (SP_B, 5), "spC": (SP_C, 7), "spD": (SP_D, 9)}
-SIPILORN_PAGE = {"spA": 16, "spB": 8, "spC": 32, "spD": 16}
+# sizes that are no multiples of 8 (width, heads' sizes, feed-forwards), a window of one token (a token sees
+# itself alone), a loop of one pass, seven heads of four channels, every expert chosen
+SP_E = model(132, 500, 1e-6, [
+    layer("parallel", pair(attn(2, 2, 40, 24, 0.15, window=1, rot=(4, 10000.0)), delta(1, 1, 44, 12, 4), 1.0, 1.0), moe(4, 4, 28)),
+    layer("delta", delta(7, 7, 4, 4, 4), dense(52)),
+    layer("delta", delta(3, 1, 20, 12, 3), moe(5, 2, 20)),
+], loop=(0, 1, 1), softcap=30.0)
+SIPILORN_CONFIGS = {"spA": (SP_A, 3), "spB": (SP_B, 5), "spC": (SP_C, 7), "spD": (SP_D, 9), "spE": (SP_E, 14)}
+SIPILORN_PAGE = {"spA": 16, "spB": 8, "spC": 32, "spD": 16, "spE": 16}
 SIPILORN_LENGTHS = {"spA": [1, 2, 12, 13, 14, 40, 61], "spB": [3, 8, 9, 17, 75, 130], "spC": [5, 69, 70, 71, 100],
-                    "spD": [1, 2, 33, 80]}
+                    "spD": [1, 2, 33, 80], "spE": [2, 35, 66]}
 
 #: factors on the drawn weights by the tensor's last name (matrices only)
 SHARP = {"q": 12.0, "k": 12.0, "v": 10.0, "g": 8.0, "o": 5.0, "b": 15.0, "a": 15.0, "up": 6.0, "down": 6.0,

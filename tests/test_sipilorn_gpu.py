@@ -16,7 +16,7 @@ from sipilorn_models import SIPILORN_LENGTHS, SIPILORN_PAGE
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-NAMES = ["spA", "spB", "spC", "spD"]
+NAMES = ["spA", "spB", "spC", "spD", "spE"]
 #: bfloat16: the share of a run's rows that may be over the tolerance, up to four times (rows at which the plain
 #: result's terms nearly cancel: an early token whose recurrence read-out is all but at right angles to its key,
 #: and the norm over the head then brings rounding up); the same rows in every way of cutting.  A window that is
