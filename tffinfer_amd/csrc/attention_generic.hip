@@ -3,7 +3,7 @@
 // the matrix-core kernels are checked against.
 //
 // One wave per (token, q head).  Keys are taken 64 at a time, one per lane:
-//   s_j = (q . k_j) * scale                   (scale after the product,
+//   s_j = (q . k_j) * scale                   (scale after the product; with a cap c > 0, s_j <- c tanh(s_j / c);
 //                                              reference paged_flash_attention.cu:723)
 //   visible iff  lo <= j <= pos               (causal: mask_op.cu:37-43; lo from the window)
 //   running max m and sum l over chunks       (paged_flash_attention.cu:746-790)
@@ -22,7 +22,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, const TC* __restrict__ k_cache,
     const TC* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
     const int32_t* __restrict__ token_req, const int32_t* __restrict__ positions, int nq, int nkv,
-    int d, int page_size, int window, float scale, const float* __restrict__ sinks) {
+    int d, int page_size, int window, float scale, const float* __restrict__ sinks, float softcap) {
     __shared__ float qs[AG_MAX_D];
     __shared__ long long voff[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -55,6 +55,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             float dot = 0.f;
             for (int e = 0; e < d; ++e) dot = fmaf(qs[e], to_f32(kp[e]), dot);
             s = dot * scale;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);      // a cap on the scores, before the mask
         }
         __syncthreads();  // earlier readers of voff are done
         voff[lane] = off;
@@ -93,7 +94,7 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out, const 
                                   const void* v_cache, const int32_t* block_tables, int bt_stride,
                                   const int32_t* token_req, const int32_t* positions, int T, int nq,
                                   int nkv, int d, int page_size, int num_pages, int window,
-                                  float scale, const float* sinks, int dtype, int cache_dtype,
+                                  float scale, const float* sinks, float softcap, int dtype, int cache_dtype,
                                   tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && token_req && positions,
                 "attention: null pointer");
@@ -113,12 +114,12 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out, const 
     if (dtype == TFF_F32)
         attention_generic_kernel<float, float><<<grid, 64, 0, s>>>(
             (const float*)q, q_stride, (float*)out, (const float*)k_cache, (const float*)v_cache,
-            block_tables, bt_stride, token_req, positions, nq, nkv, d, page_size, window, scale, sinks);
+            block_tables, bt_stride, token_req, positions, nq, nkv, d, page_size, window, scale, sinks, softcap);
     else if (dtype == TFF_BF16)
         attention_generic_kernel<bf16_t, bf16_t><<<grid, 64, 0, s>>>(
             (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache,
             (const bf16_t*)v_cache, block_tables, bt_stride, token_req, positions, nq, nkv, d,
-            page_size, window, scale, sinks);
+            page_size, window, scale, sinks, softcap);
     else
         return tff_fail("attention: unknown dtype %d", dtype);
     return tff_check_launch("attention_generic");

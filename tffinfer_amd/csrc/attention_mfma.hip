@@ -81,7 +81,14 @@ struct AttnFuse {
     // e^sink, with no key and no value: not scaled, counted once however the keys are split
     // (the kernel or merge that forms the final sum adds it).  Null: none.
     const float* sinks;
+    // A cap on the scores: s <- cap * tanh(s / cap) after the scale and before the mask.  0: none.
+    float softcap;
 };
+
+// tanh by one exponential: 1 - 2 / (1 + e^(2x)), which ends at 1 and -1 as e^(2x) overflows and vanishes.
+__device__ __forceinline__ float attn_tanh(float x) {
+    return 1.0f - 2.0f / (1.0f + __builtin_amdgcn_exp2f(x * 2.88539008177793f));
+}
 
 // RMS norm over the head and rotation of one head held as MFMA operand fragments: lane group kg
 // has the elements ks * 32 + kg * 8 .. + 7 of every 32-element step ks, so with pairs (i, i + d/2)
@@ -410,6 +417,8 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
     // rescaling 4 DT accumulator registers in every step was a quarter of them.
     const float sl2 = scale * 1.44269504088896f;
     const float slack = 8.0f / sl2;
+    // a cap c on the scores, in raw score units: s <- (c / scale) tanh(s scale / c), so that s scale is capped
+    const float cap_in = fz.softcap > 0.f ? scale / fz.softcap : 0.f, cap_out = fz.softcap > 0.f ? fz.softcap / scale : 0.f;
     int w_min_pos = c_ok ? c_pos : 0x7fffffff, w_max_lo = c_ok ? c_lo : 0;   // over the wave's columns
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -426,6 +435,11 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
                 sacc_[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[buf][kt][ks], qf[ks], sacc_[kt], 0, 0, 0); \
         float sv_[8];                                                                               \
         _Pragma("unroll") for (int e = 0; e < 8; ++e) sv_[e] = sacc_[e >> 2][e & 3];                \
+        if constexpr (DT <= 12) {   /* (the head size of 256 has no registers to spare: the host refuses a cap there) */ \
+            if (cap_in > 0.f) {                                                                     \
+                _Pragma("unroll") for (int e = 0; e < 8; ++e) sv_[e] = cap_out * attn_tanh(sv_[e] * cap_in); \
+            }                                                                                       \
+        }                                                                                           \
         if (kb_ + 31 > w_min_pos || kb_ < w_max_lo) {   /* the step touches an edge of some column (a column */ \
             /* that does not exist has a query of zeros and is masked with the others) */          \
             _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                         \
@@ -858,7 +872,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     const int32_t* __restrict__ block_tables, int bt_stride, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ start_pos, const int32_t* __restrict__ work,
     const int32_t* __restrict__ block_items, int nq, int nkv, int page_size, int page_shift,
-    int window, float scale, const float* __restrict__ sinks) {
+    int window, float scale, const float* __restrict__ sinks, float softcap) {
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KFR = 2 * KS, VFR = DT, FR = KFR + VFR;   // 1 KB fragments per slice
@@ -1009,6 +1023,8 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     // unit then has a fused multiply-add, an exponential and an addition per score to do.
     const float sl2 = scale * 1.44269504088896f;
     const float slack = 8.0f / sl2;   // 8 in the exponent's units, as a raw score
+    // a cap c on the scores, in raw score units: s <- (c / scale) tanh(s scale / c), so that s scale is capped
+    const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap > 0.f ? softcap / scale : 0.f;
     int t_min_pos[NQT], t_max_lo[NQT];
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {
@@ -1076,6 +1092,10 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
             // lane (col, g): key kb + g*8 + e is row g*4 + e%4 of tile e/4
 #pragma unroll
             for (int e = 0; e < 8; ++e) sv[e] = sacc[t][e >> 2][e & 3];
+            if (cap_in > 0.f) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sv[e] = cap_out * attn_tanh(sv[e] * cap_in);
+            }
             if (kb + 31 > t_min_pos[t] || kb < t_max_lo[t]) {   // the slice touches an edge of some column
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -1199,7 +1219,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
                        int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2,
-                       const AttnFuse* runs_only = nullptr, const float* sinks = nullptr) {
+                       const AttnFuse* runs_only = nullptr, const float* sinks = nullptr, float softcap = 0.f) {
     int page_shift = 0;   // the page size is a power of two (tff_attention_mfma_supported)
     while ((1 << page_shift) < page_size) ++page_shift;
     if (cols_per_wave == 256) {
@@ -1209,7 +1229,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         if constexpr (DT <= 8) {
             attn_mfma_block_kernel<DT, 2, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                 q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
+                block_items, nq, nkv, page_size, page_shift, window, scale, sinks, softcap);
             return tff_check_launch("attention_mfma_block256");
         } else {
             return tff_fail("attention_mfma: blocks of 256 columns take head sizes up to 128");
@@ -1224,15 +1244,15 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
             if (key_groups == 2)
                 attn_mfma_block_kernel<DT, 1, 8, 2><<<dim3(num_blocks, nkv), 1024, 0, s>>>(
                     q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                    block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
+                    block_items, nq, nkv, page_size, page_shift, window, scale, sinks, softcap);
             else
                 attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                     q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                    block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
+                    block_items, nq, nkv, page_size, page_shift, window, scale, sinks, softcap);
         } else
             attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                 q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
+                block_items, nq, nkv, page_size, page_shift, window, scale, sinks, softcap);
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, max(splits, 1));
@@ -1240,6 +1260,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
     AttnFuse fz = fuse ? *fuse : runs_only ? *runs_only
                                            : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, nullptr, nullptr};
     if (sinks) fz.sinks = sinks;
+    if (softcap > 0.f) fz.softcap = softcap;
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
@@ -1291,10 +1312,11 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const int32_t* block_items, int num_blocks,
                                int tiles_per_entry, int cols_per_wave, int key_groups, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
-                               float scale, const float* sinks, tff_stream_t stream) {
+                               float scale, const float* sinks, float softcap, tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
                 "attention_mfma: null pointer");
     TFF_REQUIRE(key_groups == 1 || key_groups == 2, "attention_mfma: %d key groups (1 or 2)", key_groups);
+    TFF_REQUIRE(!(softcap > 0.f) || d <= 192, "attention_mfma: a cap on the scores with head sizes up to 192, not %d", d);
     TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
                 "attention_mfma: %d query heads are not a multiple of %d key heads", nq, nkv);
     TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
@@ -1333,7 +1355,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                 bt_stride, cu_tokens, start_pos, work, num_work, block_items,       \
                                 num_blocks, tiles_per_entry,                                        \
                                 cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s, \
-                                nullptr, key_groups, nullptr, splits > 1 ? nullptr : sinks);
+                                nullptr, key_groups, nullptr, splits > 1 ? nullptr : sinks, softcap);
     switch (d) {
         TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
         TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)
@@ -1505,12 +1527,13 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
                                     const int32_t* key_runs, const int32_t* run_start,
                                     const int32_t* tokens, int num_runs, int num_entries, int merge,
                                     int T, int nq, int nkv, int d, int page_size, int num_pages,
-                                    int window, float scale, const float* sinks, tff_stream_t stream) {
+                                    int window, float scale, const float* sinks, float softcap, tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
                 "attention_mfma_runs: null pointer");
     TFF_REQUIRE(key_runs && run_start && tokens && part_o && part_ml,
                 "attention_mfma_runs: the runs, the tokens' rows and the workspace are needed");
     TFF_REQUIRE(((uintptr_t)key_runs % 16) == 0, "attention_mfma_runs: key_runs must be 16-byte aligned");
+    TFF_REQUIRE(!(softcap > 0.f) || d <= 192, "attention_mfma_runs: a cap on the scores with head sizes up to 192, not %d", d);
     TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
                 "attention_mfma_runs: %d query heads are not a multiple of %d key heads", nq, nkv);
     TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
@@ -1524,7 +1547,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
                 "65,535), head size %d (at most 256)", num_runs, nkv, tiles, d);
     TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && num_entries >= 0 && T >= 0, "attention_mfma_runs: bad geometry");
     if (num_entries == 0 || num_runs == 0) return 0;
-    AttnFuse fz{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, key_runs, sinks};
+    AttnFuse fz{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, key_runs, sinks, softcap > 0.f ? softcap : 0.f};
     hipStream_t s = (hipStream_t)stream;
     int rc = -1;
 #define TFF_ATTN_CASE(DTV)                                                                          \

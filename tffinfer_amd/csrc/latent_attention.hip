@@ -10,10 +10,11 @@
 // are: a key page row is [c | kr | 0 ..] up to the padded head size Dp, the (transposed) value
 // page holds c in its first kv_rank rows and zeros below.
 //
-// tff_latent_kv_store:  c = rmsnorm(x[:rank]) * w, kr = rotate(x[rank:]) into the token's slot.
+// tff_latent_kv_store:  c = rmsnorm(x[:rank]) * w, kr = rotate(x[rank:]) into the token's slot; where the
+//                       queries pass a latent vector too, its RMS norm in the same launch.
 // tff_head_linear:      out[t, h, :N] = W[h] x[t, h, :K]  (W [H, N, K]), per head, with
 //                       an optional sigmoid gate on the result and an optional tail of the
-//                       input row that is rotated by the token's position and copied behind
+//                       input row that is rotated by the token's position (either pairing) and copied behind
 //                       the product (the query's rotated part), zeros up to pad_to.
 //                       bfloat16 on the matrix cores where rows are 16-byte aligned: a wave
 //                       holds 32 tokens x 64 outputs in accumulators and reads its operands
@@ -23,14 +24,54 @@
 #include "common.h"
 #include "tffinfer_kernels.h"
 
+// Element e of the rotated part (rot elements at x, the first rot_dims of them rotated) after the rotation
+// by the position's angles cs [pair][cos, sin]: pairing 0 turns (i, i + rot_dims / 2), 1 turns (2i, 2i + 1);
+// the pair (u, w) becomes (u c - w s, w c + u s).
+template <typename T>
+__device__ __forceinline__ float latent_rotated(const T* __restrict__ x, int e, int rot_dims, int pairing,
+                                                const float* __restrict__ cs) {
+    const float v = to_f32(x[e]);
+    if (!cs || e >= rot_dims) return v;
+    int i, other;
+    bool first;
+    if (pairing == 0) {
+        const int half = rot_dims >> 1;
+        first = e < half;
+        i = first ? e : e - half;
+        other = first ? e + half : e - half;
+    } else {
+        first = !(e & 1);
+        i = e >> 1;
+        other = e ^ 1;
+    }
+    const float o = to_f32(x[other]), c = cs[2 * i], s = cs[2 * i + 1];
+    return first ? fmaf(v, c, -(o * s)) : fmaf(v, c, o * s);
+}
+
+// One block a token.  xq (may be null): the query's latent vector, q_rank elements, whose RMS norm times
+// q_norm_w goes to q_out.  x (may be null: a layer that reads another layer's cache): the key side.
 template <typename T, typename TC>
 __global__ __launch_bounds__(256) void latent_kv_store_kernel(
-    const T* __restrict__ x, int x_stride, int rank, int rot, int rot_dims,
+    const T* __restrict__ x, int x_stride, int rank, int rot, int rot_dims, int pairing,
     const float* __restrict__ norm_w, float eps, const float* __restrict__ cos_sin, int max_pos,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, TC* __restrict__ k_cache,
-    TC* __restrict__ v_cache, int page_size, int Dp) {
+    TC* __restrict__ v_cache, int page_size, int Dp, const T* __restrict__ xq, int xq_stride, int q_rank,
+    const float* __restrict__ q_norm_w, TC* __restrict__ q_out, int q_out_stride) {
     __shared__ float red[17];
     const int t = blockIdx.x, tid = threadIdx.x;
+    if (xq) {
+        const T* qr = xq + (size_t)t * xq_stride;
+        float qs = 0.f;
+        for (int e = tid; e < q_rank; e += blockDim.x) {
+            const float v = to_f32(qr[e]);
+            qs = fmaf(v, v, qs);
+        }
+        qs = block_sum(qs, red);
+        const float rq = 1.0f / sqrtf(qs / (float)q_rank + eps);
+        for (int e = tid; e < q_rank; e += blockDim.x)
+            q_out[(size_t)t * q_out_stride + e] = from_f32<TC>(to_f32(qr[e]) * rq * q_norm_w[e]);
+    }
+    if (!x) return;
     const int slot = slots[t];
     if (slot < 0) return;      // (the whole block: a token that writes no key)
     const T* xr = x + (size_t)t * x_stride;
@@ -52,43 +93,42 @@ __global__ __launch_bounds__(256) void latent_kv_store_kernel(
     int pos = positions[t];
     pos = min(max(pos, 0), max_pos - 1);
     const float* cs = cos_sin ? cos_sin + (size_t)pos * rot_dims : nullptr;   // [pair][cos, sin]
-    for (int e = tid; e < Dp - rank; e += blockDim.x) {
-        float v = 0.f;
-        if (e < rot) {
-            v = to_f32(xr[rank + e]);
-            if (cs && e < rot_dims) {
-                const int i = e >> 1;
-                const float c = cs[2 * i], s = cs[2 * i + 1];
-                const float u = to_f32(xr[rank + 2 * i]), w = to_f32(xr[rank + 2 * i + 1]);
-                v = (e & 1) ? fmaf(w, c, u * s) : fmaf(u, c, -(w * s));
-            }
-        }
-        kr[rank + e] = from_f32<TC>(v);
-    }
+    for (int e = tid; e < Dp - rank; e += blockDim.x)
+        kr[rank + e] = from_f32<TC>(e < rot ? latent_rotated<T>(xr + rank, e, rot_dims, pairing, cs) : 0.f);
 }
 
-TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, int rot, int rot_dims,
+TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, int rot, int rot_dims, int pairing,
                                 const float* norm_w, float eps, const float* cos_sin, int max_pos,
                                 const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
-                                int page_size, int num_pages, int Dp, int dtype, tff_stream_t stream) {
-    TFF_REQUIRE(x && norm_w && positions && slots && k_cache && v_cache, "latent_kv_store: null pointer");
-    TFF_REQUIRE(T >= 0 && rank > 0 && rot >= 0 && Dp >= rank + rot && x_stride >= rank + rot,
+                                int page_size, int num_pages, int Dp, const void* xq, int xq_stride, int q_rank,
+                                const float* q_norm_w, void* q_out, int q_out_stride, int dtype, int cache_dtype,
+                                tff_stream_t stream) {
+    TFF_REQUIRE(x || xq, "latent_kv_store: neither a key side nor a query side");
+    TFF_REQUIRE(!x || (norm_w && positions && slots && k_cache && v_cache), "latent_kv_store: null pointer");
+    TFF_REQUIRE(!x || (T >= 0 && rank > 0 && rot >= 0 && Dp >= rank + rot && x_stride >= rank + rot),
                 "latent_kv_store: bad sizes rank=%d rot=%d padded=%d stride=%d", rank, rot, Dp, x_stride);
-    TFF_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0 && (rot_dims == 0 || (cos_sin && max_pos > 0)),
+    TFF_REQUIRE(!x || (rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0 && (rot_dims == 0 || (cos_sin && max_pos > 0)) &&
+                       (pairing == 0 || pairing == 1)),
                 "latent_kv_store: %d rotated dimensions of %d need an even count and a table", rot_dims, rot);
-    TFF_REQUIRE(page_size > 0 && num_pages > 0, "latent_kv_store: bad cache geometry");
+    TFF_REQUIRE(!x || (page_size > 0 && num_pages > 0), "latent_kv_store: bad cache geometry");
+    TFF_REQUIRE(!xq || (q_rank > 0 && xq_stride >= q_rank && q_norm_w && q_out && q_out_stride >= q_rank),
+                "latent_kv_store: the query's latent vector of %d needs a weight and a place to go", q_rank);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == TFF_F32)
-        latent_kv_store_kernel<float, float><<<T, 256, 0, s>>>((const float*)x, x_stride, rank, rot, rot_dims, norm_w, eps,
-                                                               rot_dims ? cos_sin : nullptr, max_pos, positions, slots,
-                                                               (float*)k_cache, (float*)v_cache, page_size, Dp);
-    else if (dtype == TFF_BF16)
-        latent_kv_store_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)x, x_stride, rank, rot, rot_dims, norm_w, eps,
-                                                                 rot_dims ? cos_sin : nullptr, max_pos, positions, slots,
-                                                                 (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, Dp);
+#define TFF_LKS(TI, TCC)                                                                                              \
+    latent_kv_store_kernel<TI, TCC><<<T, 256, 0, s>>>((const TI*)x, x_stride, rank, rot, rot_dims, pairing, norm_w, eps, \
+                                                      rot_dims ? cos_sin : nullptr, max_pos, positions, slots,        \
+                                                      (TCC*)k_cache, (TCC*)v_cache, page_size, Dp, (const TI*)xq,     \
+                                                      xq_stride, q_rank, q_norm_w, (TCC*)q_out, q_out_stride)
+    if (dtype == TFF_F32 && cache_dtype == TFF_F32)
+        TFF_LKS(float, float);
+    else if (dtype == TFF_BF16 && cache_dtype == TFF_BF16)
+        TFF_LKS(bf16_t, bf16_t);
+    else if (dtype == TFF_F32 && cache_dtype == TFF_BF16)
+        TFF_LKS(float, bf16_t);
     else
-        return tff_fail("latent_kv_store: unknown dtype %d", dtype);
+        return tff_fail("latent_kv_store: rows of type %d for a cache of type %d", dtype, cache_dtype);
+#undef TFF_LKS
     return tff_check_launch("latent_kv_store");
 }
 
@@ -102,7 +142,8 @@ TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, in
 
 struct HeadLinearTail {
     int tail;            // elements of the input row behind the K multiplied ones that are copied behind the product
-    int rot_dims;        // of which the first rot_dims are rotated in pairs (2i, 2i+1)
+    int rot_dims;        // of which the first rot_dims are rotated
+    int pairing;         // 0: pairs (i, i + rot_dims / 2), 1: pairs (2i, 2i + 1)
     int pad_to;          // the output's head is filled with zeros up to this many elements
     int max_pos;
     const float* cos_sin;          // [position][pair][cos, sin], rot_dims / 2 pairs
@@ -121,12 +162,11 @@ __device__ __forceinline__ void head_tail(const T* __restrict__ x, int x_row, in
         const T* xr = x + (size_t)(t0 + tt) * x_row + (size_t)h * x_head + K;
         float v = 0.f;
         if (e < tl.tail) {
-            v = to_f32(xr[e]);
             if (e < tl.rot_dims) {
                 const int pos = min(max(tl.positions[t0 + tt], 0), tl.max_pos - 1);
-                const float* cs = tl.cos_sin + ((size_t)pos * (tl.rot_dims >> 1) + (e >> 1)) * 2;
-                const float u = to_f32(xr[e & ~1]), w = to_f32(xr[e | 1]);
-                v = (e & 1) ? fmaf(w, cs[0], u * cs[1]) : fmaf(u, cs[0], -(w * cs[1]));
+                v = latent_rotated<T>(xr, e, tl.rot_dims, tl.pairing, tl.cos_sin + (size_t)pos * tl.rot_dims);
+            } else {
+                v = to_f32(xr[e]);
             }
         }
         out[(size_t)(t0 + tt) * out_row + (size_t)h * out_head + N + e] = from_f32<T>(v);
@@ -258,7 +298,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
 
 TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt, void* out, int out_row, int out_head,
                             int T, int H, int K, int N, const void* gate, int gate_row, int tail, int rot_dims,
-                            int pad_to, const float* cos_sin, int max_pos, const int32_t* positions, int dtype,
+                            int pairing, int pad_to, const float* cos_sin, int max_pos, const int32_t* positions, int dtype,
                             tff_stream_t stream) {
     TFF_REQUIRE(x && Wt && out, "head_linear: null pointer");
     TFF_REQUIRE(T >= 0 && H > 0 && K > 0 && N > 0 && H <= 65535, "head_linear: bad sizes T=%d H=%d K=%d N=%d", T, H, K, N);
@@ -267,12 +307,13 @@ TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt
     const int width = pad_to > N ? pad_to : N;
     TFF_REQUIRE(tail >= 0 && width >= N + tail && out_head >= width && out_row >= (H - 1) * out_head + width,
                 "head_linear: output rows of %d with heads %d apart do not hold %d heads of %d", out_row, out_head, H, width);
-    TFF_REQUIRE(rot_dims >= 0 && rot_dims <= tail && rot_dims % 2 == 0 && (rot_dims == 0 || (cos_sin && positions && max_pos > 0)),
+    TFF_REQUIRE(rot_dims >= 0 && rot_dims <= tail && rot_dims % 2 == 0 && (rot_dims == 0 || (cos_sin && positions && max_pos > 0)) &&
+                (pairing == 0 || pairing == 1),
                 "head_linear: %d rotated dimensions of a tail of %d need an even count, a table and positions", rot_dims, tail);
     TFF_REQUIRE(!gate || gate_row >= H * N, "head_linear: gate rows of %d hold fewer than %d", gate_row, H * N);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    const HeadLinearTail tl{tail, rot_dims, pad_to, max_pos, cos_sin, positions};
+    const HeadLinearTail tl{tail, rot_dims, pairing, pad_to, max_pos, cos_sin, positions};
     const dim3 grid((T + HL_TT - 1) / HL_TT, H, (N + 255) / 256);
     if (dtype == TFF_F32)
         head_linear_kernel<float><<<grid, 256, 0, s>>>((const float*)x, x_row, x_head, (const float*)Wt, (float*)out, out_row,

@@ -5,7 +5,7 @@
 // partial sums, `plane` elements apart, which are added up first, plane 0, 1, ... in turn
 // (what tff_gemm leaves with keep_partials), or not at all (a layer without the sublayer).
 //
-// tff_gelu: the feed-forward's activation, exact (erf) or the tanh form, in float32.
+// tff_gelu: the feed-forward's activation, gelu exact (erf) or in the tanh form, or the square of relu, in float32.
 #include "common.h"
 #include "tffinfer_kernels.h"
 
@@ -172,17 +172,22 @@ TFF_API int tff_scale_add_rmsnorm(float* resid, const float* delta, int delta_pl
     return tff_check_launch("scale_add_rmsnorm");
 }
 
+// form 0: gelu with erf; 1: its tanh approximation; 2: the square of relu
+__device__ __forceinline__ float ffn_activation(float z, int form) {
+    if (form == 2) {
+        const float r = fmaxf(z, 0.f);
+        return r * r;
+    }
+    if (form == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+}
+
 template <typename T>
 __global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t n, int tanh_form) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const float z = to_f32(x[i]);
-    float y;
-    if (tanh_form)
-        y = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-    else
-        y = 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
-    out[i] = from_f32<T>(y);
+    out[i] = from_f32<T>(ffn_activation(z, tanh_form));
 }
 
 // bfloat16, eight elements (16 bytes) a thread
@@ -194,9 +199,7 @@ __global__ void gelu_bf16x8_kernel(const bf16_t* __restrict__ x, bf16_t* __restr
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float z = (float)a.h[j];
-        const float yv = tanh_form ? 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)))
-                                   : 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
-        b.h[j] = (bf16_t)yv;
+        b.h[j] = (bf16_t)ffn_activation(z, tanh_form);
     }
     reinterpret_cast<uint4*>(out)[i] = b.u;
 }

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(64 * RT_WAVES) void route_topk_kernel(const T* __re
     __syncthreads();
     if (wv > 0) return;
     // (one wave from here on: LDS works through its accesses in order)
-    if (softmax) {
+    if (softmax == 1) {
         // s = exp(z - max) / sum over all experts, the sum in the order of the lanes' strides and a tree
         float mx = -INFINITY;
         for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s_all[e]);
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(64 * RT_WAVES) void route_topk_kernel(const T* __re
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
         __builtin_amdgcn_wave_barrier();
     }
-    const float inv = softmax ? 1.0f : 1.0f / (sum + 1e-20f);
+    const float inv = softmax ? 1.0f : 1.0f / (sum + 1e-20f);      // (mode 2: sigmoid scores as they are)
     if (lane < top) wts[(size_t)t * top + lane] = s_all[chosen[lane]] * inv;
 }
 
@@ -176,8 +176,9 @@ template <typename T>
 __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
     const T* __restrict__ h, int h_row, const T* __restrict__ Wg, const T* __restrict__ Wu,
     const int32_t* __restrict__ idx, int top, int width, int ff, int ldw, float limit, float act_alpha, float up_offset,
-    T* __restrict__ y) {
-    // Wg null: experts without a gate, y = max(Wu h, 0)^2
+    const float* __restrict__ in_wts, T* __restrict__ y) {
+    // Wg null: experts without a gate, y = max(Wu h, 0)^2.  in_wts: the pair's weight multiplies what goes into the
+    // expert, W (w h) = w (W h): both products times w before clamps and activation.
     const int pair = blockIdx.x;                  // token * top + k
     const int t = pair / top;
     const int e = idx[pair];
@@ -187,9 +188,10 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
     const T* wu = Wu + (size_t)e * ff * ldw;
     const bool vec = sizeof(T) == 2 && width % 8 == 0 && ldw % 8 == 0 && h_row % 8 == 0 && ((uintptr_t)h % 16) == 0 &&
                      ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0;
+    const float win = in_wts ? in_wts[pair] : 1.0f;
     const int f0 = (blockIdx.y * EX_WAVES + wv) * EX_PER_WAVE;
     for (int f = f0; f < min(ff, f0 + EX_PER_WAVE); ++f) {
-        float u = row_dot<T>(hr, wu + (size_t)f * ldw, width, lane, vec);
+        float u = row_dot<T>(hr, wu + (size_t)f * ldw, width, lane, vec) * win;
         if (!wg) {
             if (lane == 0) {
                 u = fmaxf(u, 0.f);
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
             }
             continue;
         }
-        float g = row_dot<T>(hr, wg + (size_t)f * ldw, width, lane, vec);
+        float g = row_dot<T>(hr, wg + (size_t)f * ldw, width, lane, vec) * win;
         if (lane == 0) {
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
@@ -220,14 +222,15 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_down_kernel(
         for (int k = 0; k < top; ++k) {
             const int e = idx[(size_t)t * top + k];
             const float d = row_dot<T>(y + ((size_t)t * top + k) * ff, Wd + ((size_t)e * width + n) * ldw, ff, lane, vec);
-            acc = fmaf(wts[(size_t)t * top + k], d, acc);
+            acc = fmaf(wts ? wts[(size_t)t * top + k] : 1.0f, d, acc);
         }
         if (lane == 0) out[(size_t)t * width + n] = acc;
     }
 }
 
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
-                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset, void* y,
+                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset,
+                                const float* in_wts, void* y,
                                 int dtype, tff_stream_t stream) {
     TFF_REQUIRE(h && Wu && idx && y, "experts_gate_up: null pointer");
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && h_row >= width && ldw >= width,
@@ -238,11 +241,11 @@ TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const 
     TFF_REQUIRE(grid.y <= 65535, "experts_gate_up: too many outputs");
     if (dtype == TFF_F32)
         experts_gate_up_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)h, h_row, (const float*)Wg, (const float*)Wu,
-                                                                    idx, top, width, ff, ldw, limit, act_alpha, up_offset, (float*)y);
+                                                                    idx, top, width, ff, ldw, limit, act_alpha, up_offset, in_wts, (float*)y);
     else if (dtype == TFF_BF16)
         experts_gate_up_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)h, h_row, (const bf16_t*)Wg,
                                                                      (const bf16_t*)Wu, idx, top, width, ff, ldw, limit,
-                                                                     act_alpha, up_offset, (bf16_t*)y);
+                                                                     act_alpha, up_offset, in_wts, (bf16_t*)y);
     else
         return tff_fail("experts_gate_up: unknown dtype %d", dtype);
     return tff_check_launch("experts_gate_up");
@@ -250,7 +253,7 @@ TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const 
 
 TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
                              int width, int ff, int ldw, float* out, int dtype, tff_stream_t stream) {
-    TFF_REQUIRE(y && Wd && idx && wts && out, "experts_down: null pointer");
+    TFF_REQUIRE(y && Wd && idx && out, "experts_down: null pointer");      // (wts null: every pair counts 1)
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && ldw >= ff, "experts_down: bad sizes T=%d top=%d width=%d ff=%d",
                 T, top, width, ff);
     if (T == 0) return 0;
@@ -344,7 +347,9 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
     const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
     const int32_t* __restrict__ num_tiles, const float* __restrict__ wts, int T, int top, int K, int N,
     float limit, float act_alpha, float up_offset, bf16_t* __restrict__ y, float* __restrict__ out, int max_tiles, int col_blocks,
-    int ldw) {
+    int ldw, int weight_input) {
+    // weight_input: a pair's weight multiplies what goes into its expert (both first products, before clamps
+    // and activation: W (w h) = w (W h)) and the second product counts 1
     constexpr bool GATE_UP = MODE == 1;
     constexpr int ROWS = AFR * 16;       // pairs of a tile: 64, or 128 where the experts have many pairs each
     __shared__ __attribute__((aligned(16))) bf16_t lds[2 * AFR * 512];      // two sub-steps of AFR fragments
@@ -426,6 +431,7 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
 #pragma unroll
     for (int i = 0; i < AFR; ++i) {
         const int pair = tile_rows[tile * ROWS + i * 16 + r];
+        const float win = (MODE != 0 && weight_input && pair >= 0) ? wts[pair] : 1.0f;
         if (GATE_UP) {
             const float g4[4] = {acc[0][i][0], acc[0][i][1], acc[0][i][2], acc[0][i][3]};
             const float u4[4] = {acc[1][i][0], acc[1][i][1], acc[1][i][2], acc[1][i][3]};
@@ -433,8 +439,8 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
             for (int c = 0; c < 4; ++c) {
                 const int f = c0 + kg * 4 + c;
                 if (pair >= 0 && f < N) {
-                    const float gv = fminf(g4[c], limit);
-                    const float uv = fminf(fmaxf(u4[c], -limit), limit);
+                    const float gv = fminf(g4[c] * win, limit);
+                    const float uv = fminf(fmaxf(u4[c] * win, -limit), limit);
                     y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + up_offset));
                 }
             }
@@ -445,13 +451,13 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int n = c0 + j * 16 + kg * 4 + c;
-                    const float u = fmaxf(v4[c], 0.f);
+                    const float u = fmaxf(v4[c] * win, 0.f);
                     if (pair >= 0 && n < N) y[(size_t)pair * N + n] = (bf16_t)(u * u);
                 }
             }
         } else {
             const int p = max(pair, 0), t = p / top, k = p - t * top;
-            const float w = wts[p];
+            const float w = weight_input ? 1.0f : wts[p];
             float* o = out + ((size_t)k * T + t) * N;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -476,7 +482,7 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
                                  int ldw_in, int ldw_down, float limit, float act_alpha, float up_offset, int32_t* tile_expert,
                                  int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
-                                 tff_stream_t stream) {
+                                 int weight_input, tff_stream_t stream) {
     TFF_REQUIRE(h && Wu && Wd && idx && wts && tile_expert && tile_rows && num_tiles && y && out,
                 "experts_by_tiles: null pointer");
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && E <= RT_MAX_E && width > 0 && ff > 0 && h_row >= width,
@@ -502,24 +508,24 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
 #define EXT_LAUNCH(GU, AFRV, CB, ...) experts_tiles_kernel<GU, AFRV><<<((CB) + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(__VA_ARGS__)
     if (!Wg && tall)
         EXT_LAUNCH(2, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wu, nullptr, tile_expert, tile_rows,
-                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in, weight_input);
     else if (!Wg)
         EXT_LAUNCH(2, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wu, nullptr, tile_expert, tile_rows,
-                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in, weight_input);
     else if (tall)
         EXT_LAUNCH(1, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
-                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in, weight_input);
     else
         EXT_LAUNCH(1, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
-                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in, weight_input);
     rc = tff_check_launch("experts_gate_up_tiles");
     if (rc) return rc;
     if (tall)
         EXT_LAUNCH(0, 8, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
-                   T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down);
+                   T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down, weight_input);
     else
         EXT_LAUNCH(0, 4, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
-                   T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down);
+                   T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down, weight_input);
 #undef EXT_LAUNCH
     return tff_check_launch("experts_down_tiles");
 }

@@ -98,6 +98,8 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d,
 // token_req[t] names the row of block_tables; token t sees keys at positions
 // max(0, pos-window+1) .. pos of that request (window 0: from 0).
 // Works for every head size that is a multiple of 8 up to 512.
+// softcap (so for every attention entry point that takes it): c > 0 caps the scores, s <- c tanh(s / c), after the
+// scale and before the mask; 0: none.
 // sinks (float32 [nq], may be null; so for every attention entry point that takes them): a number
 // per query head whose exponential stands in the softmax's denominator beside the keys' terms,
 // with no key and no value, not scaled, counted once.
@@ -106,7 +108,7 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
                                   const int32_t* block_tables, int bt_stride,
                                   const int32_t* token_req, const int32_t* positions,
                                   int T, int nq, int nkv, int d, int page_size, int num_pages,
-                                  int window, float scale, const float* sinks, int dtype, int cache_dtype,
+                                  int window, float scale, const float* sinks, float softcap, int dtype, int cache_dtype,
                                   tff_stream_t stream);
 
 // bfloat16 attention on the matrix cores.  A wave works on `cols_per_wave` (16)
@@ -132,7 +134,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const int32_t* block_items, int num_blocks,
                                int tiles_per_entry, int cols_per_wave, int key_groups, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
-                               float scale, const float* sinks, tff_stream_t stream);
+                               float scale, const float* sinks, float softcap, tff_stream_t stream);
 // Decoding steps (every entry brings one token), bfloat16, from the fused projection's output:
 // row r of qkv ([R, (nq + 2 nkv) d], q heads first, then k, then v) is token r.  The kernel
 // does what tff_qk_norm_rope_kv and tff_attention_mfma do one after the other, in one pass:
@@ -199,7 +201,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
                                     const int32_t* key_runs, const int32_t* run_start,
                                     const int32_t* tokens, int num_runs, int num_entries, int merge,
                                     int T, int nq, int nkv, int d, int page_size, int num_pages,
-                                    int window, float scale, const float* sinks, tff_stream_t stream);
+                                    int window, float scale, const float* sinks, float softcap, tff_stream_t stream);
 
 // tff_attention_decode_fused followed by tff_attention_split_reduce, for callers that cannot
 // allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
@@ -230,10 +232,16 @@ TFF_API int tff_attention_decode_fused_static(const void* qkv, int qkv_stride, v
 // rot_dims / 2, 2]); written to the token's slot (page * page_size + offset; negative: not
 // written) of a cache of ONE key head of size Dp >= rank + rot: key row [c | kr | zeros], value
 // rows (transposed page [Dp, page_size]) c in the first rank rows.
-TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, int rot, int rot_dims,
+// pairing 0 turns the pairs (i, i + rot_dims / 2), 1 the pairs (2i, 2i + 1).  xq (may be null): rows of q_rank
+// elements, the queries' latent vectors, whose RMS norm times q_norm_w goes to q_out (rows q_out_stride apart,
+// in the cache's type).  x null: only that (a layer that reads the cache another layer fills).  dtype is the
+// rows' type, cache_dtype the cache's: the same, or float32 rows for a bfloat16 cache.
+TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, int rot, int rot_dims, int pairing,
                                 const float* norm_w, float eps, const float* cos_sin, int max_pos,
                                 const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
-                                int page_size, int num_pages, int Dp, int dtype, tff_stream_t stream);
+                                int page_size, int num_pages, int Dp, const void* xq, int xq_stride, int q_rank,
+                                const float* q_norm_w, void* q_out, int q_out_stride, int dtype, int cache_dtype,
+                                tff_stream_t stream);
 // Products per head: out[t, h * out_head + n] = sum_k x[t, h * x_head + k] * Wt[h, n, k], Wt [H, N, K].
 // gate (may be null): the result is multiplied by sigmoid(gate[t, h * N + n]).  tail > 0: the
 // `tail` elements of the input head behind the K multiplied ones are copied behind the N results,
@@ -241,7 +249,7 @@ TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, in
 // zeros up to there.
 TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt, void* out, int out_row, int out_head,
                             int T, int H, int K, int N, const void* gate, int gate_row, int tail, int rot_dims,
-                            int pad_to, const float* cos_sin, int max_pos, const int32_t* positions, int dtype,
+                            int pairing, int pad_to, const float* cos_sin, int max_pos, const int32_t* positions, int dtype,
                             tff_stream_t stream);
 
 // ---- a norm after the residual sum, and the gelu (postnorm.hip) ----
@@ -251,20 +259,46 @@ TFF_API int tff_scale_add_rmsnorm(float* resid, const float* delta, int delta_pl
                                   const float* weight, float eps, void* out, int n, int H, int out_dtype,
                                   tff_stream_t stream);
 // tanh_form 0: 0.5 z (1 + erf(z / sqrt 2)); 1: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+// (tanh_form 2: not a gelu but the square of relu, max(z, 0)^2)
 TFF_API int tff_gelu(const void* x, void* out, int64_t n, int tanh_form, int dtype, tff_stream_t stream);
+
+// ---- a norm without statistics (dyt_norm.hip) ----
+// v = resid + planes of d0 + planes of d1 (each optional); resid <- v unless rows picks rows;
+// out = tanh(alpha v) * w + b, element by element.
+TFF_API int tff_add_dyt(float* resid, const float* d0, int planes0, size_t plane0, const float* d1, int planes1,
+                        size_t plane1, float alpha, const float* w, const float* b, void* out, const int32_t* rows,
+                        int n, int W, int out_dtype, tff_stream_t stream);
+
+// ---- differential attention (diff_attention.hip) ----
+// proj float32 [T, row]: q [H, 2, D], k [G, 2, D], v [G, E] (two score maps a head), biases qb, kb, vb (may be
+// null) added, the first rot_dims elements of every map of q and k rotated (pairing as above).  q_out
+// [T, 2 H, P]: head 2 h + m holds map m at elements m D .. m D + D - 1, zeros elsewhere; the key row of kv head
+// g is [k_g0 | k_g1 | 0 ..] of P elements, the value row [v_g | 0 ..], written where slots[t] >= 0.
+TFF_API int tff_diff_qkv_store(const float* proj, size_t row, const float* qb, const float* kb, const float* vb,
+                               const float* cos_sin, int rot_dims, int pairing, int max_pos, const int32_t* positions,
+                               const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int page_size,
+                               int num_pages, int T, int H, int G, int D, int E, int P, int dtype, tff_stream_t stream);
+// a [T, a_row >= 2 H P]: the two maps' outputs of head h at (2 h) P and (2 h + 1) P, E values each.
+// out[t, h E + e] = o / sqrt(mean over the head of o^2 + eps) * out_scale * sigmoid(gate[t, h E + e]),
+// o = a_0 - lambda a_1 (gate float32, may be null).
+TFF_API int tff_diff_combine(const void* a, size_t a_row, int P, const float* gate, size_t gate_row, float lambda, float eps,
+                             float out_scale, void* out, size_t out_row, int T, int H, int E, int dtype, tff_stream_t stream);
 
 // ---- routed experts (routed_experts.hip) ----
 // Router: s = sigmoid(z), z = Wr h in float32 (Wr [E, width] float32), or z = logits [T, E] where given
 // (h and Wr may then be null); the `top` largest s + bias (bias may be null) are chosen; idx [T, top],
-// wts [T, top] = s / (sum of the chosen s + 1e-20).  softmax != 0: s = softmax(z) over all experts, wts = the chosen s.
+// wts [T, top] = s / (sum of the chosen s + 1e-20).  softmax 1: s = softmax(z) over all experts, wts = the chosen s;
+// softmax 2: s = sigmoid(z) and wts = the chosen s as they are.
 TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* logits, const float* bias, int T,
                            int width, int E, int top, int softmax, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
 // y[(t, k), :] = g * sigmoid(act_alpha * g) * (u + up_offset), g = min(Wg[e] h_t, limit), u = clamp(Wu[e] h_t, +-limit),
-// e = idx[t, k]; Wg, Wu [E, ff, width], rows ldw elements apart.
+// e = idx[t, k]; Wg, Wu [E, ff, width], rows ldw elements apart.  in_wts [T, top] (may be null): the pair's
+// weight multiplies the expert's input, that is both products before clamps and activation.
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
-                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset, void* y,
-                                int dtype, tff_stream_t stream);
+                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset,
+                                const float* in_wts, void* y, int dtype, tff_stream_t stream);
 // out[t, :] = sum_k wts[t, k] * Wd[idx[t, k]] y[(t, k), :]; Wd [E, width, ff], rows ldw elements apart; out float32.
+// wts null: every pair counts 1.
 TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
                              int width, int ff, int ldw, float* out, int dtype, tff_stream_t stream);
 
@@ -278,7 +312,7 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
                                  int ldw_in, int ldw_down, float limit, float act_alpha, float up_offset, int32_t* tile_expert,
                                  int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
-                                 tff_stream_t stream);
+                                 int weight_input, tff_stream_t stream);
 
 // ---- norms on a sublayer's output, sums over the model's depth (group_norm.hip) ----
 // y = delta row (planes added up first; row rows[r] where rows is given) cut into `groups` equal parts, each

@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 32
+ABI_VERSION = 33
 
 
 class KernelLibraryError(RuntimeError):
@@ -33,27 +33,31 @@ _SIGNATURES = {
     "tff_qk_norm_rope_kv": [_P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _P,
                             _I, _I, _I, _I, _P],
     "tff_attention_generic": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I,
-                              _F, _P, _I, _I, _P],
+                              _F, _P, _F, _I, _I, _P],
     "tff_attention_mfma_supported": [_I, _I],
     "tff_attention_mfma": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I,
-                           _I, _I, _I, _I, _I, _I, _F, _P, _P],
+                           _I, _I, _I, _I, _I, _I, _F, _P, _F, _P],
     "tff_attention_decode_fused": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
                                    _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_decode_runs": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
                                   _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_mfma_runs": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
-                                _I, _F, _P, _P],
+                                _I, _F, _P, _F, _P],
     "tff_attention_decode_fused_static": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
                                           _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_split_reduce": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P, _P],
-    "tff_latent_kv_store": [_P, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-    "tff_head_linear": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _I, _P, _I, _P],
+    "tff_latent_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P, _P, _I,
+                            _I, _I, _P],
+    "tff_head_linear": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _I, _P, _I, _P],
+    "tff_add_dyt": [_P, _P, _I, _Z, _P, _I, _Z, _F, _P, _P, _P, _P, _I, _I, _I, _P],
+    "tff_diff_qkv_store": [_P, _Z, _P, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "tff_diff_combine": [_P, _Z, _I, _P, _Z, _F, _F, _F, _P, _Z, _I, _I, _I, _I, _P],
     "tff_scale_add_rmsnorm": [_P, _P, _I, _Z, _F, _P, _F, _P, _I, _I, _I, _P],
     "tff_gelu": [_P, _P, c_int64, _I, _I, _P],
     "tff_route_topk": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
-    "tff_experts_gate_up": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _I, _P],
+    "tff_experts_gate_up": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _P, _I, _P],
     "tff_experts_tiles_supported": [_I, _I, _I],
-    "tff_experts_by_tiles": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _P, _P, _I, _P, _P, _P],
+    "tff_experts_by_tiles": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _P, _P, _I, _P, _P, _I, _P],
     "tff_group_rmsnorm_add": [_P, _P, _I, _Z, _P, _P, _I, _F, _P, _I, _I, _I, _P],
     "tff_depth_average": [_P, _Z, _I, _P, _P, _P, _Z, _I, _P],
     "tff_scale_rows": [_P, _F, _Z, _P],

@@ -444,10 +444,11 @@ def qk_norm_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int,
 def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, block_tables: torch.Tensor, token_req: torch.Tensor,
                       positions: torch.Tensor, window: int = 0, scale: float | None = None,
-                      out: torch.Tensor | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                      out: torch.Tensor | None = None, sinks: torch.Tensor | None = None,
+                      softcap: float = 0.0) -> torch.Tensor:
     """Attention of each token over its request's pages; q is [T, >= nq*d]
     with the query heads at the start of each row.  Returns [T, nq*d].
-    ``sinks`` (float32 [nq]): see :func:`paged_attention`."""
+    ``sinks`` (float32 [nq]) and ``softcap``: see :func:`paged_attention`."""
     _req(q, "attention q", ndim=2)
     T = q.shape[0]
     if q.shape[1] < nq * d:
@@ -469,7 +470,7 @@ def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch
     _lib.check(L.tff_attention_generic(
         q.data_ptr(), q.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
         block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(), positions.data_ptr(),
-        T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _ptr(sinks),
+        T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _ptr(sinks), float(softcap or 0.0),
         dtype_code(q.dtype), dtype_code(k_cache.dtype), _stream()))
     return out
 
@@ -633,7 +634,8 @@ def pick_splits(waves: int, max_context: int) -> int:
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
                    scale: float | None = None, splits: int | None = None,
                    block_bins: int | None = None, key_groups: int | None = None,
-                   block_cols: int | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                   block_cols: int | None = None, sinks: torch.Tensor | None = None,
+                   softcap: float = 0.0) -> torch.Tensor:
     """bfloat16 attention of the step's tokens on the matrix cores; decode-only
     steps split each request's keys over several waves and merge them.
     ``splits``, ``block_bins`` (blocks per kv head that share the work of
@@ -660,6 +662,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         scale = 1.0 / math.sqrt(d)
     out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
     _check_sinks(sinks, nq)
+    softcap = float(softcap or 0.0)
     L = _lib.load()
     stream = _stream()
 
@@ -674,7 +677,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
             v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
             batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks, tiles, cols,
             groups, splits, R if splits > 1 else T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window),
-            float(scale), _ptr(sinks), stream))
+            float(scale), _ptr(sinks), softcap, stream))
         if splits > 1:
             _lib.check(L.tff_attention_split_reduce(
                 part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R, nq, d, _ptr(rows),
@@ -693,7 +696,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
                 v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
                 runs.data_ptr(), kv.run_start.data_ptr(), batch.cu_tokens.data_ptr(), runs.shape[0], R,
                 1 if kv.runs_merge else 0, T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale),
-                _ptr(sinks), stream))
+                _ptr(sinks), softcap, stream))
             return out
         if splits is None:
             splits = pick_splits(R * tiles * nkv, batch.max_context)
@@ -731,7 +734,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
                 q.data_ptr(), q.stride(0), out.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), k_cache.data_ptr(),
                 v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
                 runs.data_ptr(), run_start.data_ptr(), tokens.data_ptr(), runs.shape[0], len(single), 1 if merge else 0,
-                T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _ptr(sinks), stream))
+                T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _ptr(sinks), softcap, stream))
         else:
             work = _attention_work(batch, G, 16, q.device, "single")
             if "single_rows" not in cache:
@@ -887,17 +890,20 @@ def qkv_attention(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weig
 
 
 def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
-                    scale: float | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                    scale: float | None = None, sinks: torch.Tensor | None = None,
+                    softcap: float = 0.0) -> torch.Tensor:
     """Attention of a step's tokens over the cache view ``kv`` (k_cache,
     v_cache, block_tables) with the step's ``batch``.  bfloat16 with a head
     size the matrix-core kernel takes runs there; everything else (float32,
     other head sizes) on the general kernel.  ``sinks`` (float32 [nq]): a
     number per query head whose exponential is one more term of the softmax's
-    denominator, with no key and no value, not scaled."""
-    if mfma_attention_supported(q.dtype, d, kv.k_cache.shape[2]):
-        return attention_mfma(q, nq, nkv, d, kv, batch, window, scale, sinks=sinks)
+    denominator, with no key and no value, not scaled.  ``softcap`` c > 0: the
+    scaled scores are capped, s <- c tanh(s / c), before the mask."""
+    # (the matrix-core kernels cap scores at head sizes up to 192)
+    if mfma_attention_supported(q.dtype, d, kv.k_cache.shape[2]) and not (softcap and d > 192):
+        return attention_mfma(q, nq, nkv, d, kv, batch, window, scale, sinks=sinks, softcap=softcap)
     return attention_generic(q, nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
-                             batch.token_req, batch.positions, window, scale, sinks=sinks)
+                             batch.token_req, batch.positions, window, scale, sinks=sinks, softcap=softcap)
 
 
 MFMA_HEAD_SIZES = tuple(range(16, 129, 16)) + (192, 256)
@@ -914,52 +920,78 @@ def padded_head_size(d: int, dtype: torch.dtype) -> int:
     return -(-d // 8) * 8
 
 
-def latent_kv_store(x: torch.Tensor, rank: int, rot: int, norm_w: torch.Tensor, eps: float,
+def latent_kv_store(x: torch.Tensor | None, rank: int, rot: int, norm_w: torch.Tensor | None, eps: float,
                     cos_sin: torch.Tensor | None, positions: torch.Tensor, slot_mapping: torch.Tensor,
-                    k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
-    """Rows x [T, >= rank + rot] (rows may be strided): the RMS norm of the first ``rank`` elements
-    times ``norm_w`` and the next ``rot`` elements, rotated by ``cos_sin`` [max_pos, dims / 2, 2]
-    in pairs (2i, 2i+1), go to the tokens' slots of a cache of one key head of the padded size
-    (keys [pages, 1, page_size, Dp], values transposed)."""
-    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
-        raise _lib.KernelError("latent_kv_store x: expected a GPU matrix with unit inner stride")
-    T = x.shape[0]
-    if x.shape[1] < rank + rot:
-        raise _lib.KernelError(f"latent_kv_store: rows of {x.shape[1]} hold fewer than {rank} + {rot}")
-    _req(norm_w, "latent norm weight", torch.float32, 1)
-    if norm_w.numel() != rank:
-        raise _lib.KernelError(f"latent norm weight: {norm_w.numel()} elements for a rank of {rank}")
-    _req(k_cache, "k cache", x.dtype, 4)
-    _req(v_cache, "v cache", x.dtype, 4)
+                    k_cache: torch.Tensor, v_cache: torch.Tensor, pairing: int = 1,
+                    q_latent: torch.Tensor | None = None, q_norm_w: torch.Tensor | None = None) -> torch.Tensor | None:
+    """Rows x [T, >= rank + rot] (rows may be strided; float32 rows may go to a bfloat16 cache): the RMS norm of
+    the first ``rank`` elements times ``norm_w`` and the next ``rot`` elements, rotated by ``cos_sin``
+    [max_pos, dims / 2, 2] in pairs (2i, 2i+1) (``pairing`` 1) or (i, i + dims/2) (``pairing`` 0), go to the
+    tokens' slots of a cache of one key head of the padded size (keys [pages, 1, page_size, Dp], values
+    transposed).  ``q_latent`` [T, q_rank] (rows may be strided, x's type): the queries' latent vectors, whose
+    RMS norm times ``q_norm_w`` is returned in the cache's type, from the same launch.  ``x`` None: only
+    that (a layer that reads a cache another layer fills)."""
+    _req(k_cache, "k cache", ndim=4)
+    _req(v_cache, "v cache", k_cache.dtype, 4)
     Dp = k_cache.shape[3]
     _check_cache(k_cache, v_cache, 1, Dp, "latent_kv_store")
-    if Dp < rank + rot:
-        raise _lib.KernelError(f"latent_kv_store: a cache of head size {Dp} does not hold {rank} + {rot}")
+    src = x if x is not None else q_latent
+    if src is None:
+        raise _lib.KernelError("latent_kv_store: neither rows for the cache nor latent vectors of queries")
+    T = src.shape[0]
+    for t, nm in ((x, "x"), (q_latent, "q_latent")):
+        if t is not None and (not isinstance(t, torch.Tensor) or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1
+                              or t.dtype != src.dtype or t.shape[0] != T):
+            raise _lib.KernelError(f"latent_kv_store {nm}: expected a GPU matrix with unit inner stride, one row a token")
+    if src.dtype != k_cache.dtype and not (src.dtype == torch.float32 and k_cache.dtype == torch.bfloat16):
+        raise _lib.KernelError(f"latent_kv_store: rows of {src.dtype} for a cache of {k_cache.dtype}")
     dims, max_pos = 0, 0
-    if cos_sin is not None:
-        _req(cos_sin, "rotation table", torch.float32, 3)
-        max_pos, dims = cos_sin.shape[0], 2 * cos_sin.shape[1]
-        if cos_sin.shape[2] != 2 or dims > rot:
-            raise _lib.KernelError(f"rotation table {tuple(cos_sin.shape)} does not fit a rotated part of {rot}")
-    _req(positions, "positions", torch.int32, 1)
-    _req(slot_mapping, "slot_mapping", torch.int32, 1)
-    if positions.numel() != T or slot_mapping.numel() != T:
-        raise _lib.KernelError("latent_kv_store: positions and slot_mapping need one entry per token")
+    if x is not None:
+        if x.shape[1] < rank + rot:
+            raise _lib.KernelError(f"latent_kv_store: rows of {x.shape[1]} hold fewer than {rank} + {rot}")
+        _req(norm_w, "latent norm weight", torch.float32, 1)
+        if norm_w.numel() != rank:
+            raise _lib.KernelError(f"latent norm weight: {norm_w.numel()} elements for a rank of {rank}")
+        if Dp < rank + rot:
+            raise _lib.KernelError(f"latent_kv_store: a cache of head size {Dp} does not hold {rank} + {rot}")
+        if cos_sin is not None:
+            _req(cos_sin, "rotation table", torch.float32, 3)
+            max_pos, dims = cos_sin.shape[0], 2 * cos_sin.shape[1]
+            if cos_sin.shape[2] != 2 or dims > rot:
+                raise _lib.KernelError(f"rotation table {tuple(cos_sin.shape)} does not fit a rotated part of {rot}")
+        _req(positions, "positions", torch.int32, 1)
+        _req(slot_mapping, "slot_mapping", torch.int32, 1)
+        if positions.numel() != T or slot_mapping.numel() != T:
+            raise _lib.KernelError("latent_kv_store: positions and slot_mapping need one entry per token")
+    q_out, q_rank = None, 0
+    if q_latent is not None:
+        q_rank = q_latent.shape[1]
+        _req(q_norm_w, "query latent norm weight", torch.float32, 1)
+        if q_norm_w.numel() != q_rank:
+            raise _lib.KernelError(f"query latent norm weight: {q_norm_w.numel()} elements for a rank of {q_rank}")
+        q_out = torch.empty(T, q_rank, dtype=k_cache.dtype, device=src.device)
+
+    def row(t):
+        return t.stride(0) if T > 1 else t.shape[1]
+
     _lib.check(_lib.load().tff_latent_kv_store(
-        x.data_ptr(), x.stride(0) if T > 1 else x.shape[1], T, int(rank), int(rot), dims, norm_w.data_ptr(), float(eps),
-        _ptr(cos_sin), max_pos, positions.data_ptr(), slot_mapping.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-        k_cache.shape[2], k_cache.shape[0], Dp, dtype_code(x.dtype), _stream()))
+        _ptr(x), row(x) if x is not None else 0, T, int(rank), int(rot), dims, int(pairing), _ptr(norm_w), float(eps),
+        _ptr(cos_sin) if x is not None else None, max_pos, _ptr(positions), _ptr(slot_mapping), k_cache.data_ptr(),
+        v_cache.data_ptr(), k_cache.shape[2], k_cache.shape[0], Dp, _ptr(q_latent), row(q_latent) if q_latent is not None else 0,
+        q_rank, _ptr(q_norm_w), _ptr(q_out), q_rank, dtype_code(src.dtype), dtype_code(k_cache.dtype), _stream()))
+    return q_out
 
 
 def head_linear(x: torch.Tensor, x_head: int, weight_t: torch.Tensor, out_head: int | None = None,
                 gate: torch.Tensor | None = None, tail: int = 0, cos_sin: torch.Tensor | None = None,
-                positions: torch.Tensor | None = None) -> torch.Tensor:
+                positions: torch.Tensor | None = None, pairing: int = 1) -> torch.Tensor:
     """Products per head: x [T, >= H * x_head] (head h starts at h * x_head; rows may be strided),
     ``weight_t`` [H, N, K]: out[t, h, :N] = weight_t[h] x[t, h, :K].  Returns [T, H * out_head]
     (``out_head`` >= N + tail, by default N + tail), zeros behind what is written.
     ``gate`` [T, >= H * N] (rows may be strided): the products are multiplied by its sigmoid.
     ``tail``: so many elements of the input head behind the K are copied behind the products, the
-    first ``2 * cos_sin.shape[1]`` of them rotated in pairs (2i, 2i+1) by the tokens' positions."""
+    first ``2 * cos_sin.shape[1]`` of them rotated by the tokens' positions, in pairs (2i, 2i+1)
+    (``pairing`` 1) or (i, i + dims/2) (``pairing`` 0)."""
     if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
         raise _lib.KernelError("head_linear x: expected a GPU matrix with unit inner stride")
     _req(weight_t, "head_linear weight", x.dtype, 3)
@@ -987,7 +1019,7 @@ def head_linear(x: torch.Tensor, x_head: int, weight_t: torch.Tensor, out_head: 
     out = torch.empty(T, H * out_head, dtype=x.dtype, device=x.device)
     _lib.check(_lib.load().tff_head_linear(
         x.data_ptr(), x.stride(0) if T > 1 else x.shape[1], int(x_head), weight_t.data_ptr(), out.data_ptr(),
-        H * out_head, out_head, T, H, K, N, _ptr(gate), gate_row, int(tail), dims, out_head if out_head > N else 0,
+        H * out_head, out_head, T, H, K, N, _ptr(gate), gate_row, int(tail), dims, int(pairing), out_head if out_head > N else 0,
         _ptr(cos_sin) if dims else None, max_pos, _ptr(positions) if dims else None, dtype_code(x.dtype), _stream()))
     return out
 
@@ -1029,12 +1061,21 @@ def gelu(x: torch.Tensor, tanh_form: bool = False) -> torch.Tensor:
     return out
 
 
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    """max(z, 0)^2, element by element, in float32."""
+    _req(x, "relu_squared input")
+    out = torch.empty_like(x)
+    _lib.check(_lib.load().tff_gelu(x.data_ptr(), out.data_ptr(), x.numel(), 2, dtype_code(x.dtype), _stream()))
+    return out
+
+
 def route_topk(h: torch.Tensor | None, router: torch.Tensor | None, bias: torch.Tensor | None, top: int,
-               logits: torch.Tensor | None = None, softmax: bool = False):
+               logits: torch.Tensor | None = None, softmax: bool = False, normalize: bool = True):
     """s = sigmoid(z) with z = h . router^T in float32 (router float32 [E, width]) or z = ``logits``
     (float32 [T, E], a product that ran before); the ``top`` experts with the largest s + bias;
     returns (int32 [T, top], float32 [T, top] = s / (sum of the chosen s + 1e-20)).  With
-    ``softmax``, s = softmax(z) over all experts and the weights are the chosen s as they are."""
+    ``softmax``, s = softmax(z) over all experts and the weights are the chosen s as they are; without
+    ``normalize``, s = sigmoid(z) and the weights are the chosen s as they are."""
     if logits is not None:
         _req(logits, "router logits", torch.float32, 2)
         T, E = logits.shape
@@ -1055,7 +1096,7 @@ def route_topk(h: torch.Tensor | None, router: torch.Tensor | None, bias: torch.
     wts = torch.empty(T, top, dtype=torch.float32, device=dev)
     _lib.check(_lib.load().tff_route_topk(None if logits is not None else h.data_ptr(), width,
                                           None if logits is not None else router.data_ptr(), _ptr(logits), _ptr(bias),
-                                          T, width, E, int(top), 1 if softmax else 0, idx.data_ptr(), wts.data_ptr(), dtype_code(dt), _stream()))
+                                          T, width, E, int(top), 1 if softmax else (0 if normalize else 2), idx.data_ptr(), wts.data_ptr(), dtype_code(dt), _stream()))
     return idx, wts
 
 
@@ -1076,10 +1117,12 @@ EXPERT_TILES_MIN_TOKENS = 32
 
 def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                    idx: torch.Tensor, wts: torch.Tensor, limit: float, act_alpha: float,
-                   by_tiles: bool | None = None, up_offset: float = 1.0) -> torch.Tensor:
+                   by_tiles: bool | None = None, up_offset: float = 1.0, weight_input: bool = False) -> torch.Tensor:
     """The weighted sum of each token's chosen experts: y = g sigmoid(act_alpha g) (u + up_offset) with
     g = min(Wg h, limit), u = clamp(Wu h, -limit, limit); out = sum_k wts[:, k] Wd y.
-    ``w_gate`` None: experts without a gate, y = max(Wu h, 0)^2.
+    ``w_gate`` None: experts without a gate, y = max(Wu h, 0)^2.  ``weight_input``: a pair's weight multiplies
+    what goes into its expert instead of what comes out, out = sum_k expert_k(wts[:, k] h); since W (w h) = w (W h)
+    it is applied to both first products, before clamps and activation.
     ``w_gate``, ``w_up`` [E, ff, >= width], ``w_down`` [E, width, >= ff] of h's type (the last
     dimension may be wider than what is multiplied: see :func:`pad_expert_rows`).  float32
     [T, width], or (many tokens in bfloat16, ``by_tiles``) [top, T, width]: the terms of the sum
@@ -1113,13 +1156,13 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
         _lib.check(L.tff_experts_by_tiles(
             h.data_ptr(), width, _ptr(w_gate), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(),
             T, top, E, width, ff, ld_in, ld_down, float(limit), float(act_alpha), float(up_offset), tables.data_ptr(), tables[max_tiles:].data_ptr(),
-            tables[129 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), _stream()))
+            tables[129 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), 1 if weight_input else 0, _stream()))
         return out if top > 1 else out[0]
     _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, _ptr(w_gate), w_up.data_ptr(), idx.data_ptr(), T, top, E,
-                                     width, ff, ld_in, float(limit), float(act_alpha), float(up_offset), y.data_ptr(), dtype_code(h.dtype),
-                                     _stream()))
+                                     width, ff, ld_in, float(limit), float(act_alpha), float(up_offset),
+                                     wts.data_ptr() if weight_input else None, y.data_ptr(), dtype_code(h.dtype), _stream()))
     out = torch.empty(T, width, dtype=torch.float32, device=h.device)
-    _lib.check(L.tff_experts_down(y.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(), T, top, E, width, ff,
+    _lib.check(L.tff_experts_down(y.data_ptr(), w_down.data_ptr(), idx.data_ptr(), None if weight_input else wts.data_ptr(), T, top, E, width, ff,
                                   ld_down, out.data_ptr(), dtype_code(h.dtype), _stream()))
     return out
 
@@ -1541,6 +1584,87 @@ def sigmoid_gate_heads(o: torch.Tensor, o_head: int, g: torch.Tensor, H: int, E:
     return out
 
 
+def add_dyt(resid: torch.Tensor, delta, alpha: float, weight: torch.Tensor, bias: torch.Tensor,
+            out_dtype: torch.dtype, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """``resid += delta`` (``delta``: None, what a mixer or feed-forward returned, or :class:`PendingTerms`; not
+    added when ``rows`` is given) and the norm without statistics of the sum, tanh(alpha v) * weight + bias element
+    by element; with ``rows`` (int32) the norm of those rows only, ``resid`` untouched."""
+    _req(resid, "add_dyt resid", torch.float32, 2)
+    H = resid.shape[1]
+    for w, nm in ((weight, "weight"), (bias, "bias")):
+        _req(w, f"add_dyt {nm}", torch.float32, 1)
+        if w.numel() != H:
+            raise _lib.KernelError(f"add_dyt: {nm} has {w.numel()} elements, rows have {H}")
+    terms = delta.terms if isinstance(delta, PendingTerms) else ([] if delta is None else [delta])
+    d = [_planes_of(t, resid.shape, "add_dyt term") for t in terms] + [(None, 0, 0)] * 2
+    if rows is not None:
+        _req(rows, "add_dyt rows", torch.int32, 1)
+        n = rows.numel()
+    else:
+        n = resid.shape[0]
+    out = torch.empty(n, H, dtype=out_dtype, device=resid.device)
+    _lib.check(_lib.load().tff_add_dyt(resid.data_ptr(), _ptr(d[0][0]), d[0][1], d[0][2], _ptr(d[1][0]), d[1][1], d[1][2],
+                                       float(alpha), weight.data_ptr(), bias.data_ptr(), out.data_ptr(), _ptr(rows), n, H,
+                                       dtype_code(out_dtype), _stream()))
+    return out
+
+
+def diff_qkv_store(proj: torch.Tensor, H: int, G: int, D: int, E: int, q_bias, k_bias, v_bias,
+                   cos_sin: torch.Tensor | None, pairing: int, positions: torch.Tensor, kv) -> torch.Tensor:
+    """The projections of a differential attention, ``proj`` float32 [T, >= 2 H D + 2 G D + G E] = q [H, 2, D],
+    k [G, 2, D], v [G, E] (rows may be strided), with their biases (float32, or None) added and the first
+    ``2 * cos_sin.shape[1]`` elements of every map of q and k rotated.  Returns the queries [T, 2 H P] in the
+    cache's type, P the cache's head size: head 2 h + m holds map m at elements m D .. m D + D - 1 and zeros
+    elsewhere.  The token's key row [k_g0 | k_g1 | 0 ..] and value row [v_g | 0 ..] go to its slot of ``kv``."""
+    cols = 2 * H * D + 2 * G * D + G * E
+    T = proj.shape[0]
+    row = _rows2(proj, "diff_qkv_store proj", torch.float32, cols)
+    k_cache, v_cache = kv.k_cache, kv.v_cache
+    _req(k_cache, "k cache", ndim=4)
+    _req(v_cache, "v cache", k_cache.dtype, 4)
+    P = k_cache.shape[3]
+    _check_cache(k_cache, v_cache, G, P, "diff_qkv_store")
+    if P < 2 * D or P < E:
+        raise _lib.KernelError(f"diff_qkv_store: a cache head of {P} does not hold two maps of {D} or values of {E}")
+    for b, n, nm in ((q_bias, 2 * H * D, "q bias"), (k_bias, 2 * G * D, "k bias"), (v_bias, G * E, "v bias")):
+        if b is not None:
+            _req(b, nm, torch.float32, 1)
+            if b.numel() != n:
+                raise _lib.KernelError(f"diff_qkv_store: {nm} of {b.numel()} elements, expected {n}")
+    dims, max_pos = 0, 0
+    if cos_sin is not None:
+        _req(cos_sin, "rotation table", torch.float32, 3)
+        max_pos, dims = cos_sin.shape[0], 2 * cos_sin.shape[1]
+        if cos_sin.shape[2] != 2 or dims > D:
+            raise _lib.KernelError(f"rotation table {tuple(cos_sin.shape)} does not fit a map of {D}")
+    _req(positions, "positions", torch.int32, 1)
+    _req(kv.slot_mapping, "slot_mapping", torch.int32, 1)
+    if positions.numel() < T or kv.slot_mapping.numel() < T:
+        raise _lib.KernelError("diff_qkv_store: positions and slot_mapping need one entry per token")
+    q = torch.empty(T, 2 * H * P, dtype=k_cache.dtype, device=proj.device)
+    _lib.check(_lib.load().tff_diff_qkv_store(
+        proj.data_ptr(), row, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(cos_sin), dims, int(pairing), max_pos,
+        positions.data_ptr(), kv.slot_mapping.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        k_cache.shape[2], k_cache.shape[0], T, H, G, D, E, P, dtype_code(k_cache.dtype), _stream()))
+    return q
+
+
+def diff_combine(a: torch.Tensor, P: int, gate: torch.Tensor | None, lam: float, eps: float, out_scale: float,
+                 H: int, E: int) -> torch.Tensor:
+    """``a`` [T, 2 H P]: the outputs of a head's two score maps side by side (E values each at the start of their
+    P).  o = a_0 - lam a_1; returns o / sqrt(mean over the head of o^2 + eps) * out_scale * sigmoid(gate), [T, H E]
+    in a's type.  ``gate`` float32 [T, >= H E] (rows may be strided) or None."""
+    T = a.shape[0]
+    a_row = _rows2(a, "diff_combine a", a.dtype, 2 * H * P)
+    gate_row = _rows2(gate, "diff_combine gate", torch.float32, H * E) if gate is not None else 0
+    if gate is not None and gate.shape[0] != T:
+        raise _lib.KernelError("diff_combine: the gate needs one row per token")
+    out = torch.empty(T, H * E, dtype=a.dtype, device=a.device)
+    _lib.check(_lib.load().tff_diff_combine(a.data_ptr(), a_row, int(P), _ptr(gate), gate_row, float(lam), float(eps),
+                                            float(out_scale), out.data_ptr(), H * E, T, H, E, dtype_code(a.dtype), _stream()))
+    return out
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """``silu(gate) * up`` for gate_up [T, 2I] = [gate | up]."""
     _req(gate_up, "swiglu input", ndim=2)
@@ -1677,6 +1801,10 @@ OP_TABLE = {
     "head_linear": head_linear,
     "scale_add_rmsnorm": scale_add_rmsnorm,
     "gelu": gelu,
+    "relu_squared": relu_squared,
+    "add_dyt": add_dyt,
+    "diff_qkv_store": diff_qkv_store,
+    "diff_combine": diff_combine,
     "route_topk": route_topk,
     "routed_experts": routed_experts,
     "cast": cast,

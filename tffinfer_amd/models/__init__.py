@@ -1,4 +1,4 @@
-from . import disunex, netovik, qwen3, sipilorn  # noqa: F401  (registers the architectures)
+from . import disunex, netovik, qwen3, rutevik, sipilorn  # noqa: F401  (registers the architectures)
 from .decoder import DecoderModel, TensorNames
 from .registry import (Architecture, build_model_skeleton, config_from_dict, get_architecture,
                        load_config, load_model, register_architecture, registered_architectures)

@@ -106,7 +106,8 @@ class DecoderModel:
                                  f"{self.stream_offsets.rows if self.stream_offsets else 0}")
         self.final_norm = NORMS.build(config.final_norm_spec())
         self.head = OutputHead(V, H, self.embedding if config.tie_word_embeddings else None,
-                               softcap=getattr(config, "logit_softcap", None))
+                               softcap=getattr(config, "logit_softcap", None),
+                               scale=getattr(config, "logit_scale", None))
 
     # ---- weights ---------------------------------------------------------
     def _weighted_parts(self):

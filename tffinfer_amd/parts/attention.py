@@ -220,3 +220,112 @@ class GatedGQAttention(Mixer):
         if self.external_output:
             raise RuntimeError("gated attention: its output matrix was left to a combining mixer")
         return ctx.ops.linear(self.forward_inner(ctx, x), self.w_o, out_dtype=torch.float32, partials=True)
+
+
+@register_mixer("differential_attention")
+class DifferentialAttention(Mixer):
+    """Grouped-query attention in which every head has two score maps over the same values, and the
+    second map's output is subtracted from the first's:
+
+        q_hm = rot((Wq x + bq)_hm),  k_gm = rot((Wk x + bk)_gm)    (m = 0, 1; maps of ``head_dim``)
+        v_g  = (Wv x + bv)_g                                        (heads of ``value_dim``)
+        s_hm(i, j) = scale * q_hm(i) . k_gm(j),  capped to softcap * tanh(s / softcap) where there is a cap
+        a_hm(i) = sum over j <= i of softmax_j(s_hm(i, .)) v_g(j),   g = h // (heads / kv_heads)
+        lambda  = exp(lq1 . lk1) - exp(lq2 . lk2) + diff            (one number for the layer)
+        o_h = a_h0 - lambda a_h1;   o_h <- o_h / sqrt(mean(o_h^2) + eps) * (1 - diff)
+        out = Wo [o_h * sigmoid(Wg x)_h]_h
+
+    q and k are laid out head by head as [map 0 | map 1]; rot: the position encoding, on as many
+    elements of every map as it rotates.  ``bias`` False: no bq, bk, bv; ``output_gate`` False: no gate.
+
+    The attention proper runs on the paged kernels of ``GQAttention`` as 2 heads a head on ``kv_heads``
+    kv heads: a key row holds both maps' keys side by side, a query is zero outside its own map's part,
+    so the two maps share one stored key row and one stored value row.  The cache's head size is the
+    larger of 2 ``head_dim`` and ``value_dim``, brought up to a size those kernels take.  All four
+    projections are one product whose result stays float32 until biases and rotation are done.
+    """
+
+    graph_safe = True
+    input_goes_to_linear = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                 position, scale: float | None = None, softcap: float | None = None, diff: float = 0.0,
+                 norm_eps: float = 1e-6, bias: bool = True, output_gate: bool = True):
+        self.hidden_size = int(hidden_size)
+        self.num_heads = int(num_heads)
+        self.num_kv_heads = int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        self.value_dim = int(value_dim)
+        if min(self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim) <= 0:
+            raise ConfigError("differential attention: sizes must be positive")
+        if self.num_heads % self.num_kv_heads:
+            raise ConfigError(f"differential attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.softcap = float(softcap) if softcap else 0.0
+        if self.softcap < 0:
+            raise ConfigError("differential attention: the cap on the scores must not be negative")
+        self.diff = float(diff)
+        self.norm_eps = float(norm_eps)
+        self.has_bias = bool(bias)
+        self.has_gate = bool(output_gate)
+        if isinstance(position, PartSpec):
+            position = POSITION_ENCODINGS.build(position)
+        if position is not None and not isinstance(position, PositionEncoding):
+            raise ConfigError("differential attention: 'position' must be a position encoding or its spec")
+        if position is not None and position.rotary_dim > self.head_dim:
+            raise ConfigError(f"differential attention: {position.rotary_dim} rotated elements of a map of {self.head_dim}")
+        self.position = position
+        self._dtype = torch.bfloat16
+        self.w_in = self.w_o = self.q_bias = self.k_bias = self.v_bias = None
+        self.lam = 0.0
+
+    # ---- sizes -----------------------------------------------------------
+    def padded_head_dim(self) -> int:
+        from ..kernels.ops import padded_head_size
+        return padded_head_size(max(2 * self.head_dim, self.value_dim), self._dtype)
+
+    def cache_spec(self):
+        return KVCacheSpec(self.num_kv_heads, self.padded_head_dim())
+
+    def flops_per_query_key_pair(self):
+        return 4 * 2 * self.num_heads * self.padded_head_dim()
+
+    def weight_specs(self):
+        W, H, G, D, E = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        specs = {"q": WeightSpec((H * 2 * D, W)), "k": WeightSpec((G * 2 * D, W)), "v": WeightSpec((G * E, W)),
+                 "o": WeightSpec((W, H * E))}
+        if self.has_bias:
+            specs |= {"q.b": WeightSpec((H * 2 * D,), "norm_offset"), "k.b": WeightSpec((G * 2 * D,), "norm_offset"),
+                      "v.b": WeightSpec((G * E,), "norm_offset")}
+        for n in ("lq1", "lk1", "lq2", "lk2"):
+            specs[n] = WeightSpec((D,), "norm_offset")
+        if self.has_gate:
+            specs["g"] = WeightSpec((H * E, W))
+        return specs
+
+    def load_weights(self, weights, dtype, device):
+        self._dtype = dtype
+        kind = weights["q"].dtype
+        stacked = [weights["q"], weights["k"], weights["v"]] + ([weights["g"]] if self.has_gate else [])
+        self.w_in = to_device(torch.cat([w.to(kind) for w in stacked], 0), dtype, device)
+        self.w_o = to_device(weights["o"], dtype, device)
+        f32 = lambda n: weights[n].to(torch.float32).contiguous().to(device)  # noqa: E731
+        if self.has_bias:
+            self.q_bias, self.k_bias, self.v_bias = f32("q.b"), f32("k.b"), f32("v.b")
+        # one number for the layer, formed once, in float32
+        l = {n: weights[n].to(torch.float32) for n in ("lq1", "lk1", "lq2", "lk2")}
+        self.lam = float(torch.exp((l["lq1"] * l["lk1"]).sum()) - torch.exp((l["lq2"] * l["lk2"]).sum())
+                         + torch.tensor(self.diff, dtype=torch.float32))
+
+    def forward(self, ctx, x):
+        ops, kv, b = ctx.ops, ctx.kv, ctx.batch
+        H, G, D, E = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        P = kv.k_cache.shape[3]
+        proj = ops.linear(x, self.w_in, out_dtype=torch.float32)
+        table = self.position.cached_table(ctx.max_positions, proj.device) if self.position is not None else None
+        pairing = 1 if (self.position is not None and self.position.pairing == "interleaved") else 0
+        q = ops.diff_qkv_store(proj, H, G, D, E, self.q_bias, self.k_bias, self.v_bias, table, pairing, b.positions, kv)
+        a = ops.paged_attention(q, 2 * H, G, P, kv, b, 0, self.scale, softcap=self.softcap)
+        gate = proj[:, 2 * H * D + 2 * G * D + G * E:] if self.has_gate else None
+        o = ops.diff_combine(a, P, gate, self.lam, self.norm_eps, 1.0 - self.diff, H, E)
+        return ops.linear(o, self.w_o, out_dtype=torch.float32, partials=True)

@@ -20,10 +20,14 @@ class PreNormBlock(Block):
     def __init__(self, mixer, feed_forward, make_norm):
         self.norm1 = make_norm()
         self.mixer = mixer
-        self.norm2 = make_norm()
         self.feed_forward = feed_forward
+        # (a layer without a feed-forward has no second sum and no second norm)
+        self.has_ffn = not getattr(feed_forward, "is_none", False)
+        self.norm2 = make_norm() if self.has_ffn else None
 
     def children(self):
+        if not self.has_ffn:
+            return {"norm1": self.norm1, "mixer": self.mixer}
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
                 "feed_forward": self.feed_forward}
 
@@ -37,6 +41,8 @@ class PreNormBlock(Block):
     def forward(self, ctx, resid, pending):
         h = self._norm(self.norm1, self.mixer, ctx, resid, pending)
         a = self.mixer.forward(ctx, h)
+        if not self.has_ffn:
+            return a
         z = self._norm(self.norm2, self.feed_forward, ctx, resid, a)
         return self.feed_forward.forward(ctx, z)
 

@@ -42,15 +42,18 @@ class OutputHead(Part):
     """logits = y . Wout^T in float32, no bias, no scale
     (src/core/model/qwen3/QWen3Creator.cpp:161-165, :324-329).  With tied
     embeddings the head has no tensor of its own and uses the embedding's.
-    ``softcap`` c: the logits leave as c * tanh(logits / c)."""
+    ``softcap`` c: the logits leave as c * tanh(logits / c).  ``scale``: the logits are multiplied by it
+    (in float32, before a cap)."""
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Embedding | None, softcap: float | None = None):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Embedding | None, softcap: float | None = None,
+                 scale: float | None = None):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
         self.tied_to = tied_to
         self.softcap = float(softcap) if softcap else 0.0
+        self.scale = float(scale) if scale is not None else 1.0
         self._weight = None
 
     def weight_specs(self):
@@ -68,4 +71,6 @@ class OutputHead(Part):
 
     def forward(self, ctx, y):
         logits = ctx.ops.linear(y, self.weight, out_dtype=torch.float32)
+        if self.scale != 1.0:
+            ctx.ops.scale_rows(logits, self.scale)
         return ctx.ops.softcap_(logits, self.softcap) if self.softcap else logits

@@ -73,16 +73,21 @@ class NoFeedForward(FeedForward):
 
 @register_feed_forward("gelu_mlp")
 class GeluMLP(FeedForward):
-    """f = Wdown gelu(Wup z), no gate and no biases; the gelu is the exact one,
-    0.5 z (1 + erf(z / sqrt 2)), or with ``tanh_form`` its tanh approximation."""
+    """f = Wdown act(Wup z), no gate and no biases.  ``activation`` "gelu": the exact one,
+    0.5 z (1 + erf(z / sqrt 2)), or with ``tanh_form`` its tanh approximation; "relu2": the
+    square of relu, max(z, 0)^2."""
 
     graph_safe = True
     input_goes_to_linear = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, tanh_form: bool = False):
+    def __init__(self, hidden_size: int, intermediate_size: int, tanh_form: bool = False, activation: str = "gelu"):
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.tanh_form = bool(tanh_form)
+        self.activation = str(activation)
+        if self.activation not in ("gelu", "relu2"):
+            from ..config.base import ConfigError
+            raise ConfigError(f"feed-forward: unknown activation '{activation}' (gelu, relu2)")
         self.w_up = self.w_down = None
 
     def weight_specs(self):
@@ -94,7 +99,8 @@ class GeluMLP(FeedForward):
         self.w_down = to_device(weights["down"], dtype, device)
 
     def forward(self, ctx, x):
-        a = ctx.ops.gelu(ctx.ops.linear(x, self.w_up), self.tanh_form)
+        u = ctx.ops.linear(x, self.w_up)
+        a = ctx.ops.relu_squared(u) if self.activation == "relu2" else ctx.ops.gelu(u, self.tanh_form)
         return ctx.ops.linear(a, self.w_down, out_dtype=torch.float32, partials=True)
 
 
@@ -110,7 +116,10 @@ class RoutedExperts(FeedForward):
         f = sum over the chosen e of w_e f_e
 
     ``router_softmax``: s = softmax(Wr z) over all experts instead, and w_e = s_e as it is.
+    ``normalize`` False: w_e = s_e as it is (the sigmoid's scores, not made to add up to one).
     ``limit`` None: no clamp; ``up_offset`` 0 and ``act_alpha`` 1: y = silu(g) * u.
+    ``weight_input``: the weight multiplies what goes into the expert, f = sum of expert_e(w_e z),
+    instead of what comes out.
 
     The experts' matrices lie stacked, [experts, out, in], so that a kernel finds an expert's
     rows by its number."""
@@ -119,8 +128,11 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
                  limit: float | None, act_alpha: float = 1.702, correction: bool = True,
-                 router_softmax: bool = False, up_offset: float = 1.0):
+                 router_softmax: bool = False, up_offset: float = 1.0, normalize: bool = True,
+                 weight_input: bool = False):
         self.router_softmax = bool(router_softmax)
+        self.normalize = bool(normalize)
+        self.weight_input = bool(weight_input)
         self.up_offset = float(up_offset)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
@@ -181,11 +193,12 @@ class RoutedExperts(FeedForward):
         if self.router_w is not None:
             idx, wts = ops.route_topk(None, None, self.correction, self.top,
                                       logits=ops.linear(x, self.router_w, out_dtype=torch.float32),
-                                      softmax=self.router_softmax)
+                                      softmax=self.router_softmax, normalize=self.normalize)
         else:
-            idx, wts = ops.route_topk(x, self.router, self.correction, self.top, softmax=self.router_softmax)
+            idx, wts = ops.route_topk(x, self.router, self.correction, self.top, softmax=self.router_softmax,
+                                      normalize=self.normalize)
         return ops.routed_experts(x, self.w_gate, self.w_up, self.w_down, idx, wts, self.limit, self.act_alpha,
-                                  up_offset=self.up_offset)
+                                  up_offset=self.up_offset, weight_input=self.weight_input)
 
 
 @register_feed_forward("table_experts")

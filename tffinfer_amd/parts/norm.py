@@ -1,4 +1,4 @@
-"""RMS norm on the residual stream."""
+"""Norms on the residual stream: RMS norms, and a norm without statistics."""
 from __future__ import annotations
 
 import torch
@@ -95,3 +95,30 @@ class GroupRMSNorm(Norm):
         if delta is not None:
             resid += ctx.ops.as_tensor(delta)
         return ctx.ops.group_rmsnorm_add(None, resid, self.weight, self.groups, self.eps, ctx.act_dtype, rows=rows)
+
+
+@register_norm("dyt")
+class DynamicTanh(Norm):
+    """A norm that computes no mean and no variance: y = tanh(alpha * v) * w + b element by element,
+    with one learned scalar ``alpha`` and vectors ``w`` and ``b`` of the row's size; v is the residual
+    stream plus the term still pending.  float32 throughout.  The tensors are called ``weight``, ``b``
+    and ``alpha`` (a tensor without dimensions)."""
+
+    graph_safe = True
+
+    def __init__(self, size: int):
+        self.size = int(size)
+        self.weight = self.bias = None
+        self.alpha = 1.0
+
+    def weight_specs(self):
+        return {"weight": WeightSpec((self.size,), "norm"), "b": WeightSpec((self.size,), "norm_offset"),
+                "alpha": WeightSpec((), "unit_interval")}
+
+    def load_weights(self, weights, dtype, device):
+        self.weight = weights["weight"].to(torch.float32).contiguous().to(device)
+        self.bias = weights["b"].to(torch.float32).contiguous().to(device)
+        self.alpha = float(weights["alpha"].to(torch.float32))      # (a kernel argument: read once, at load)
+
+    def forward(self, ctx, resid, delta, rows=None, for_linear=False):
+        return ctx.ops.add_dyt(resid, delta, self.alpha, self.weight, self.bias, ctx.act_dtype, rows=rows)

@@ -70,3 +70,33 @@ class RotaryEmbedding(PositionEncoding):
             t = torch.stack([torch.cos(a), torch.sin(a)], -1).to(torch.float32).contiguous().to(device)
             _TABLES[key] = t
         return t
+
+
+@register_position_encoding("rope_scaled")
+class ScaledRotaryEmbedding(RotaryEmbedding):
+    """The rotation whose long waves are slowed down so that a model reaches beyond the length it
+    first learned: with f = theta^(-2i/rot) and the wave's length l = 2 pi / f,
+
+        l < original / high:   f as it is
+        l > original / low:    f / factor
+        between:               (1 - s) f / factor + s f,   s = (original / l - low) / (high - low).
+
+    ``factor``, ``low``, ``high`` and ``original`` (a length in tokens) are parameters."""
+
+    def __init__(self, head_dim: int, theta: float, factor: float, low: float, high: float, original: float,
+                 pairing: str = "half", rotary_dim: int | None = None):
+        super().__init__(head_dim, theta, pairing, rotary_dim)
+        self.factor, self.low, self.high, self.original = float(factor), float(low), float(high), float(original)
+        if not (self.factor > 0 and self.high > self.low >= 0 and self.original > 0):
+            raise ConfigError(f"scaled rope: factor {factor}, low {low}, high {high}, original {original} "
+                              "(positive, and high above low)")
+
+    def angles(self, max_positions: int) -> torch.Tensor:
+        half = self.rotary_dim // 2
+        i = torch.arange(half, dtype=torch.float64)
+        f = torch.exp(-(2.0 * i / self.rotary_dim) * math.log(self.theta))
+        wave = 2.0 * math.pi / f
+        s = (self.original / wave - self.low) / (self.high - self.low)
+        mid = (1.0 - s) * f / self.factor + s * f
+        f = torch.where(wave < self.original / self.high, f, torch.where(wave > self.original / self.low, f / self.factor, mid))
+        return torch.arange(max_positions, dtype=torch.float64)[:, None] * f[None, :]
