@@ -45,6 +45,14 @@ def sipilorn_dirs(tmp_path_factory):
     return {name: make_sipilorn_dir(str(base / name), cfg, seed) for name, (cfg, seed) in SIPILORN_CONFIGS.items()}
 
 
+@pytest.fixture(scope="session")
+def rutevik_dirs(tmp_path_factory):
+    """Model folders of the tiny Rutevik configurations (sharpened weights), once per session."""
+    from rutevik_models import RUTEVIK_CONFIGS, make_rutevik_dir
+    base = tmp_path_factory.mktemp("rutevik")
+    return {name: make_rutevik_dir(str(base / name), cfg, seed) for name, (cfg, seed) in RUTEVIK_CONFIGS.items()}
+
+
 @pytest.fixture(autouse=True)
 def _seeded():
     """Every test draws the same random inputs in every run."""

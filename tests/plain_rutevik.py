@@ -147,13 +147,13 @@ def routed_experts(m: dict, P: dict, h: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def router_margin(m: dict, P: dict, h: torch.Tensor) -> float:
-    """The smallest gap between a token's last chosen score and its first rejected one."""
+def router_margins(m: dict, P: dict, h: torch.Tensor) -> torch.Tensor:
+    """Per token, the gap between its last chosen score and its first rejected one."""
     top, E = m["router"]["top"], m["router"]["experts"]
     if top >= E:
-        return math.inf
+        return torch.full((h.shape[0],), math.inf, dtype=h.dtype)
     s = torch.sort(sigmoid(h @ P["router"].T), -1, descending=True).values
-    return float((s[:, top - 1] - s[:, top]).min())
+    return s[:, top - 1] - s[:, top]
 
 
 def feed_forward(m, P: dict, h: torch.Tensor):
@@ -187,7 +187,7 @@ def norm(P: dict, name: str, x: torch.Tensor) -> torch.Tensor:
 
 def forward(cfg: dict, P: dict, tokens: list, streams: list | None = None, margins: list | None = None) -> torch.Tensor:
     """float64 logits [T, vocab] of a whole sequence; ``streams`` collects the stream after every
-    layer, ``margins`` the routers' smallest gaps."""
+    layer, ``margins`` every router's gaps, a tensor [T] per mixture of experts."""
     eps = cfg["norm"]["eps"]
     x = P["embed"][torch.tensor(tokens)]
     caches = {}
@@ -209,7 +209,7 @@ def forward(cfg: dict, P: dict, tokens: list, streams: list | None = None, margi
         if L.get("mlp") is not None:
             z = norm(W, "norm2", x)
             if margins is not None and L["mlp"]["kind"] == "moe":
-                margins.append(router_margin(L["mlp"], sub(W, "mlp."), z))
+                margins.append(router_margins(L["mlp"], sub(W, "mlp."), z))
             x = x + feed_forward(L["mlp"], sub(W, "mlp."), z)
         if streams is not None:
             streams.append(x.clone())

@@ -1,0 +1,240 @@
+"""The Rutevik configuration: what its config.json turns into, what is refused, which layer calls share a
+cache, the rotation with slowed-down long waves, and properties of the plain implementation (all on the CPU)."""
+import copy
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import plain_rutevik as plain
+from rutevik_models import RUTEVIK_CONFIGS, RV_A, RV_B, RV_C, RV_D, make_rutevik_dir
+from tffinfer_amd.config.base import ConfigError, LayerCall
+from tffinfer_amd.models import build_model_skeleton, config_from_dict, load_config
+from tffinfer_amd.parts import (DifferentialAttention, DynamicTanh, GeluMLP, KVCacheSpec, LatentAttention, NoFeedForward,
+                                PreNormBlock, RoutedExperts, ScaledRotaryEmbedding)
+from tffinfer_amd.weights.loader import WeightError, check_weights
+from tffinfer_amd.weights.safetensors_io import load_model_dir
+
+
+def test_every_size_and_constant_comes_from_the_file():
+    cfg = config_from_dict(copy.deepcopy(RV_A))
+    model = build_model_skeleton(cfg)
+    assert [type(b) for b in model.blocks] == [PreNormBlock] * 4
+    assert [type(b.mixer) for b in model.blocks] == [LatentAttention, DifferentialAttention, LatentAttention, LatentAttention]
+    assert [type(b.feed_forward) for b in model.blocks] == [GeluMLP, RoutedExperts, RoutedExperts, NoFeedForward]
+    a = model.blocks[0].mixer
+    assert (a.num_heads, a.head_dim, a.rot_dim, a.value_dim, a.kv_rank, a.q_rank, a.scale) == (3, 16, 8, 24, 40, 24, 0.2)
+    assert (a.latent_norm_eps, a.window, a.has_sink, a.has_gate, a.shared_cache) == (1e-6, 0, False, False, False)
+    assert (a.position.rotary_dim, a.position.theta, a.position.pairing) == (8, 10000.0, "half")
+    assert a.cache_spec() == KVCacheSpec(1, 48)
+    r = model.blocks[2].mixer
+    assert r.shared_cache and (r.num_heads, r.head_dim, r.value_dim, r.q_rank) == (2, 24, 16, 32) and r.cache_spec() == a.cache_spec()
+    d = model.blocks[1].mixer
+    assert (d.num_heads, d.num_kv_heads, d.head_dim, d.value_dim, d.scale, d.softcap, d.diff, d.norm_eps) == \
+        (4, 2, 16, 24, 0.3, 5.0, 0.2, 1e-6)
+    assert isinstance(d.position, ScaledRotaryEmbedding)
+    assert (d.position.rotary_dim, d.position.theta, d.position.factor, d.position.low, d.position.high, d.position.original) == \
+        (8, 500.0, 4.0, 1.0, 2.0, 32.0)
+    assert d.cache_spec() == KVCacheSpec(2, 32)         # two maps of 16 side by side, values of 24
+    ff = model.blocks[0].feed_forward
+    assert (ff.intermediate_size, ff.activation) == (72, "relu2")
+    ex = model.blocks[1].feed_forward
+    assert (ex.num_experts, ex.top, ex.intermediate_size) == (5, 2, 24)
+    assert (ex.normalize, ex.weight_input, ex.has_correction, ex.router_softmax, ex.act_alpha, ex.up_offset) == \
+        (False, True, False, False, 1.0, 0.0) and ex.limit == float("inf")
+    assert isinstance(model.final_norm, DynamicTanh) and model.final_norm.size == 64
+    assert model.head.scale == 0.5 and model.head.softcap == 0.0 and model.head.tied_to is None
+    # another file: other constants, a scale of 1, no cap, no scaling, kv heads that default to the heads
+    b = build_model_skeleton(config_from_dict(copy.deepcopy(RV_B)))
+    assert b.head.scale == 1.0 and b.blocks[0].mixer.softcap == 0.0 and not isinstance(b.blocks[0].mixer.position, ScaledRotaryEmbedding)
+    assert b.blocks[0].mixer.cache_spec() == KVCacheSpec(1, 64) and b.blocks[2].mixer.cache_spec() == KVCacheSpec(6, 16)
+    m = copy.deepcopy(RV_B)
+    del m["layers"][2]["mixer"]["kv_heads"], m["layers"][2]["mixer"]["vdim"], m["logit_scale"]
+    c = build_model_skeleton(config_from_dict(m))
+    assert (c.blocks[2].mixer.num_kv_heads, c.blocks[2].mixer.value_dim, c.head.scale) == (6, 8, 1.0)
+
+
+def test_which_layer_calls_share_a_cache():
+    """A layer with kv_from works on the cache of the layer it names and writes nothing there; the cache manager
+    gives the two one set of pages."""
+    from tffinfer_amd.cache.manager import CacheManager
+    assert config_from_dict(copy.deepcopy(RV_A)).layer_schedule() == [
+        LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 0, False), LayerCall(3, 0, False)]
+    assert config_from_dict(copy.deepcopy(RV_B)).layer_schedule() == [LayerCall(i, i) for i in range(3)]
+    assert config_from_dict(copy.deepcopy(RV_C)).layer_schedule() == [
+        LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2), LayerCall(3, 2, False), LayerCall(4, 0, False)]
+    model = build_model_skeleton(config_from_dict(copy.deepcopy(RV_C)))
+    needs = model.call_requirements()
+    cache = CacheManager(needs, page_size=32, num_pages=24, max_seqs=2)
+    # three caches for five layer calls; the attention's (one kv head of 32) and the second latent one (a key of
+    # 22 + 10) ask for pages of one shape and share a pool
+    assert sorted(cid for g in cache.groups for cid in g.cache_ids) == [0, 1, 2]
+    assert sorted(tuple(g.cache_ids) for g in cache.groups) == [(0,), (1, 2)]
+    cache.add_request("a")
+    cache.reserve("a", 100)
+    cache.commit("a", 100)
+    cache.check()
+    cache.release("a")
+    assert all(g.pool.num_used == 0 for g in cache.groups)
+
+
+def test_tensor_names_follow_the_files():
+    names = build_model_skeleton(config_from_dict(copy.deepcopy(RV_A))).expected_tensors()
+    for n in ("embed", "final.norm", "final.norm.b", "final.norm.alpha", "head", "l0.norm1", "l0.norm1.b", "l0.norm1.alpha",
+              "l0.norm2", "l0.mix.dq", "l0.mix.dq.norm", "l0.mix.uq", "l0.mix.dkv", "l0.mix.dkv.norm", "l0.mix.uk", "l0.mix.uv",
+              "l0.mix.o", "l0.mlp.up", "l0.mlp.down", "l1.mix.q", "l1.mix.q.b", "l1.mix.k", "l1.mix.k.b", "l1.mix.v", "l1.mix.v.b",
+              "l1.mix.lq1", "l1.mix.lk1", "l1.mix.lq2", "l1.mix.lk2", "l1.mix.g", "l1.mix.o", "l1.mlp.router", "l1.mlp.e0.gate",
+              "l1.mlp.e4.down", "l2.mix.dq", "l2.mix.uk", "l3.norm1"):
+        assert n in names, n
+    assert not any(n in names for n in ("l2.mix.dkv", "l2.mix.dkv.norm", "l3.mix.dkv", "l0.mix.q", "l0.mix.g", "l0.mix.sink",
+                                        "l1.mlp.correction", "l0.mlp.gate", "l3.mlp.up"))
+    assert names["l3.norm2"].optional and names["l3.norm2.alpha"].optional and not names["l0.norm2"].optional
+    assert names["l0.norm1.alpha"].shape == () and names["l0.norm1.b"].shape == (64,)
+    assert names["l0.mix.dq"].shape == (24, 64) and names["l0.mix.uq"].shape == (3 * 24, 24) and names["l0.mix.dkv"].shape == (48, 64)
+    assert names["l0.mix.uk"].shape == (48, 40) and names["l0.mix.uv"].shape == (72, 40) and names["l0.mix.o"].shape == (64, 72)
+    assert names["l1.mix.q"].shape == (4 * 2 * 16, 64) and names["l1.mix.k"].shape == (2 * 2 * 16, 64)
+    assert names["l1.mix.v"].shape == (48, 64) and names["l1.mix.g"].shape == (96, 64) and names["l1.mix.lq1"].shape == (16,)
+
+
+def test_round_trip_and_refusals(tmp_path):
+    d = make_rutevik_dir(str(tmp_path / "m"), RV_A, 1, sharp=False)
+    cfg = load_config(d)
+    back = cfg.to_dict()
+    assert back["layers"] == RV_A["layers"] and back["logit_scale"] == 0.5
+    assert config_from_dict(json.loads(json.dumps(back))).layer_schedule() == cfg.layer_schedule()
+    found = load_model_dir(d)
+    names = build_model_skeleton(cfg).expected_tensors()
+    check_weights(names, found, set(), d)
+    assert "l3.norm2" not in found and found["l0.norm1.alpha"].shape == ()
+    # a file that holds the second norm of a layer without a feed-forward all the same is taken
+    found["l3.norm2"], found["l3.norm2.b"], found["l3.norm2.alpha"] = found["l0.norm2"], found["l0.norm2.b"], found["l0.norm2.alpha"]
+    check_weights(names, found, set(), d)
+    del found["l1.mix.k.b"]
+    with pytest.raises(WeightError) as e:
+        check_weights(names, found, set(), d)
+    assert e.value.missing == ["l1.mix.k.b"]
+    for breaker, text in (
+            (lambda c: c["layers"][0].update(type="other"), "mixer"),
+            (lambda c: c["layers"][1]["mlp"].update(kind="sparse"), "feed-forward"),
+            (lambda c: c["layers"][0]["mixer"].pop("scale"), "scale"),
+            (lambda c: c["layers"][0]["mixer"].pop("q_rank"), "q_rank"),
+            (lambda c: c["layers"][1]["mixer"].pop("diff"), "diff"),
+            (lambda c: c["layers"][1]["mixer"].update(kv_heads=3), "kv heads"),
+            (lambda c: c["layers"][1]["mixer"]["rot"].update(dims=20), "dims"),
+            (lambda c: c["layers"][1]["mixer"]["rot"]["scaling"].pop("original"), "original"),
+            (lambda c: c["layers"][1]["mixer"]["rot"]["scaling"].update(high=0.5), "high"),
+            (lambda c: c["layers"][2]["mixer"].update(kv_from=1), "latent attention"),
+            (lambda c: c["layers"][2]["mixer"].update(kv_from=2), "another"),
+            (lambda c: c["layers"][3]["mixer"].update(kv_from=2), "of its own"),
+            (lambda c: c["layers"][0]["mixer"].update(kv_from=2), "of its own"),
+            (lambda c: c["layers"][2]["mixer"].update(kv_rank=32), "equal"),
+            (lambda c: c["layers"][2]["mixer"]["rot"].update(base=5.0), "equal"),
+            (lambda c: c["layers"][1]["mixer"].update(kv_from=0), "only a latent attention"),
+            (lambda c: c.pop("norm"), "norm"),
+            (lambda c: c.pop("width"), "width"),
+            (lambda c: c["layers"][1]["mlp"]["router"].update(top=9), "top")):
+        bad = copy.deepcopy(RV_A)
+        breaker(bad)
+        with pytest.raises(ConfigError) as e:
+            build_model_skeleton(config_from_dict(bad))
+        assert text in str(e.value), (text, str(e.value))
+
+
+@pytest.mark.parametrize("dims,base,scaling", [(8, 500.0, (4.0, 1.0, 2.0, 32)), (64, 1e4, (8.0, 1.0, 4.0, 64)),
+                                               (32, 1e6, (8.0, 1.0, 4.0, 8192)), (4, 1e4, (2.0, 1.0, 3.0, 16))])
+def test_the_rotation_with_slowed_down_long_waves(dims, base, scaling):
+    """The engine's table holds cos and sin of position times the plain implementation's frequencies: short waves
+    as they are, long waves slower by the factor, and the ones between on the way from one to the other."""
+    enc = ScaledRotaryEmbedding(dims + 8, base, *scaling, rotary_dim=dims)
+    table = enc.table(50, "cpu")
+    sc = dict(zip(("factor", "low", "high", "original"), scaling))
+    f = plain.frequencies(dims, base, sc)
+    ang = torch.arange(50, dtype=torch.float64)[:, None] * f[None, :]
+    assert table.shape == (50, dims // 2, 2)
+    assert torch.allclose(table[..., 0].double(), torch.cos(ang), atol=1e-6) and torch.allclose(table[..., 1].double(), torch.sin(ang), atol=1e-6)
+    plain_f = plain.frequencies(dims, base)
+    wave = 2 * math.pi / plain_f
+    assert torch.equal(f[wave < sc["original"] / sc["high"]], plain_f[wave < sc["original"] / sc["high"]])
+    slow = wave > sc["original"] / sc["low"]
+    assert torch.allclose(f[slow], plain_f[slow] / sc["factor"])
+    between = ~slow & ~(wave < sc["original"] / sc["high"])
+    assert bool(((f[between] <= plain_f[between]) & (f[between] >= plain_f[between] / sc["factor"])).all())
+    # another parameter is another table
+    other = ScaledRotaryEmbedding(dims + 8, base, scaling[0] * 2, *scaling[1:], rotary_dim=dims)
+    assert other.table_key() != enc.table_key()
+
+
+def test_the_plain_pieces():
+    x = torch.ones(3, 1, 6, dtype=torch.float64)
+    y = plain.rotate(x, plain.frequencies(4, 100.0))
+    assert torch.equal(y[0], x[0]) and torch.equal(y[..., 4:], x[..., 4:])
+    a = torch.tensor(2.0, dtype=torch.float64)
+    assert torch.allclose(y[2, 0, 0], torch.cos(a) - torch.sin(a)) and torch.allclose(y[2, 0, 2], torch.cos(a) + torch.sin(a))
+    assert torch.allclose(y[2, 0, 1], torch.cos(a / 10) - torch.sin(a / 10))
+    p = plain.causal_softmax(torch.zeros(4, 4, dtype=torch.float64))
+    assert torch.allclose(p[2], torch.tensor([1 / 3, 1 / 3, 1 / 3, 0.0], dtype=torch.float64))
+    z = torch.tensor([-2.0, 0.0, 3.0], dtype=torch.float64)
+    assert torch.allclose(plain.dense_ff({"up": torch.eye(3, dtype=torch.float64), "down": torch.eye(3, dtype=torch.float64)}, z[None])[0],
+                          torch.tensor([0.0, 0.0, 9.0], dtype=torch.float64))
+    assert torch.allclose(plain.dyt(z, 0.5, torch.full((3,), 2.0, dtype=torch.float64), torch.ones(3, dtype=torch.float64)),
+                          2 * torch.tanh(z / 2) + 1)
+    # one expert of two, chosen by the larger score; its weight goes in, not out
+    P = {"router": torch.tensor([[1.0, 0.0], [0.0, 1.0]], dtype=torch.float64)}
+    for e in range(2):
+        P[f"e{e}.gate"] = P[f"e{e}.up"] = torch.eye(2, dtype=torch.float64) * (e + 1)
+        P[f"e{e}.down"] = torch.eye(2, dtype=torch.float64)
+    h = torch.tensor([[0.5, 2.0]], dtype=torch.float64)
+    s = plain.sigmoid(torch.tensor(2.0, dtype=torch.float64))
+    zin = 2 * s * h[0]
+    assert torch.allclose(plain.routed_experts({"router": {"top": 1, "experts": 2}}, P, h)[0], plain.silu(zin) * zin)
+
+
+def test_the_test_configurations_differ_from_each_other():
+    seen = set()
+    for name, (cfg, _) in RUTEVIK_CONFIGS.items():
+        key = (cfg["width"], cfg["vocab"], cfg["norm"]["eps"], len(cfg["layers"]))
+        assert key not in seen
+        seen.add(key)
+    assert RV_B["logit_scale"] == 1.0 and RV_B["layers"][0]["type"] == "attention" and RV_D["layers"][0]["type"] == "attention"
+    assert not any("kv_from" in L["mixer"] for L in RV_B["layers"])
+    assert os.path.basename(__file__).startswith("test_")
+
+
+@pytest.mark.parametrize("name", ["rvA", "rvC"])
+def test_the_sharpened_weights_show_a_lost_cache_a_wrong_map_and_a_wrong_source(tmp_path, name):
+    """What the comparisons on the GPU rest on: in the plain implementation itself, a request that goes on without its
+    earlier tokens, a reader that takes its own layer's input for the borrowed cache's, and a second map that is
+    left out each move some row of logits by more than four times (the map: twice) what any row may differ by in
+    bfloat16."""
+    from helpers import rel_err, tol
+    from rutevik_models import clear_tokens
+    cfg, seed = RUTEVIK_CONFIGS[name]
+    d = make_rutevik_dir(str(tmp_path / name), cfg, seed)
+    c, P = plain.load(d)
+    toks = list(clear_tokens(d, 90, c["vocab"], 5))
+    ref = plain.forward(c, P, toks)
+    limit = 4 * tol("bfloat16", name)
+    tail = plain.forward(c, P, toks[50:])
+    assert max(rel_err(tail[i], ref[50 + i]) for i in range(len(tail))) > limit
+    # a reader whose source is another layer's cache of the same shape
+    readers = [i for i, L in enumerate(c["layers"]) if "kv_from" in L["mixer"]]
+    i = readers[-1]
+    wrong = copy.deepcopy(c)
+    src = c["layers"][i]["mixer"]["kv_from"]
+    for k in ("dkv", "dkv.norm"):
+        P[f"l{i}.mix.{k}"] = P[f"l{src}.mix.{k}"]
+    del wrong["layers"][i]["mixer"]["kv_from"]          # (its own input through the same matrices, not the source's cache)
+    out = plain.forward(wrong, P, toks)
+    assert max(rel_err(out[t], ref[t]) for t in range(len(toks))) > limit
+    # no second map: lambda's part gone
+    j = next(n for n, L in enumerate(c["layers"]) if L["type"] == "attention")
+    P2 = dict(P)
+    P2[f"l{j}.mix.lq1"] = P[f"l{j}.mix.lq1"] * 0 - 50.0
+    P2[f"l{j}.mix.lk1"] = P[f"l{j}.mix.lk1"] * 0 + 1.0
+    P2[f"l{j}.mix.lq2"], P2[f"l{j}.mix.lk2"] = P2[f"l{j}.mix.lq1"], P2[f"l{j}.mix.lk1"]
+    flat = copy.deepcopy(c)
+    flat["layers"][j]["mixer"]["diff"] = 0.0            # lambda = e^-big - e^-big + 0 = 0
+    out = plain.forward(flat, P2, toks)
+    assert max(rel_err(out[t], ref[t]) for t in range(len(toks))) > limit / 2

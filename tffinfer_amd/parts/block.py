@@ -21,13 +21,14 @@ class PreNormBlock(Block):
         self.norm1 = make_norm()
         self.mixer = mixer
         self.feed_forward = feed_forward
-        # (a layer without a feed-forward has no second sum and no second norm)
+        # (a layer without a feed-forward has no second sum; a second norm that a file holds all the same is
+        # not run)
         self.has_ffn = not getattr(feed_forward, "is_none", False)
-        self.norm2 = make_norm() if self.has_ffn else None
+        self.norm2 = make_norm()
+        if not self.has_ffn:
+            self.norm2.optional = True
 
     def children(self):
-        if not self.has_ffn:
-            return {"norm1": self.norm1, "mixer": self.mixer}
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
                 "feed_forward": self.feed_forward}
 

@@ -102,20 +102,26 @@ class DynamicTanh(Norm):
     """A norm that computes no mean and no variance: y = tanh(alpha * v) * w + b element by element,
     with one learned scalar ``alpha`` and vectors ``w`` and ``b`` of the row's size; v is the residual
     stream plus the term still pending.  float32 throughout.  The tensors are called ``weight``, ``b``
-    and ``alpha`` (a tensor without dimensions)."""
+    and ``alpha`` (a tensor without dimensions).  ``optional``: a file may leave them out (the norm of
+    a sublayer that a layer does not have); the norm then has no weight and is not to be run."""
 
     graph_safe = True
 
-    def __init__(self, size: int):
+    def __init__(self, size: int, optional: bool = False):
         self.size = int(size)
+        self.optional = bool(optional)
         self.weight = self.bias = None
         self.alpha = 1.0
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.size,), "norm"), "b": WeightSpec((self.size,), "norm_offset"),
-                "alpha": WeightSpec((), "unit_interval")}
+        return {"weight": WeightSpec((self.size,), "norm", optional=self.optional),
+                "b": WeightSpec((self.size,), "norm_offset", optional=self.optional),
+                "alpha": WeightSpec((), "unit_interval", optional=self.optional)}
 
     def load_weights(self, weights, dtype, device):
+        if not all(k in weights for k in ("weight", "b", "alpha")):
+            self.weight = self.bias = None
+            return
         self.weight = weights["weight"].to(torch.float32).contiguous().to(device)
         self.bias = weights["b"].to(torch.float32).contiguous().to(device)
         self.alpha = float(weights["alpha"].to(torch.float32))      # (a kernel argument: read once, at load)

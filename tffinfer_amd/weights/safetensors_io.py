@@ -152,5 +152,6 @@ def save_file(tensors: dict[str, torch.Tensor], path: str, metadata: dict | None
         f.write(raw)
         for name in order:
             t = tensors[name].detach().cpu().contiguous()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            # (a tensor without dimensions is stored as its one element)
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")
     os.replace(tmp, path)
