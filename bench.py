@@ -110,8 +110,40 @@ SIPILORN_SHAPES = {
                       dim=128, window=1024, pair_heads=8, dense_ff=12288, experts=32, top=4, expert_ff=3072)),
 }
 
+def rutevik_shape(width, heads, dim, rot, vdim, rank, q_rank, diff_heads, diff_kv_heads, diff_dim, diff_vdim, dense_ff,
+                  experts, top, expert_ff, layers, vocab=151936):
+    """A Rutevik configuration of ``layers`` layers: a latent attention that fills its cache, one that reads it,
+    then a differential attention, and so on; dense feed-forwards and mixtures of experts in turn."""
+    def latent(source):
+        m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "q_rank": q_rank,
+             "scale": (dim + rot) ** -0.5, "rot": {"base": 20000.0, "dims": rot}}
+        if source is not None:
+            m["kv_from"] = source
+        return {"type": "latent_attention", "mixer": m}
+    diff = {"type": "attention", "mixer": {
+        "heads": diff_heads, "kv_heads": diff_kv_heads, "dim": diff_dim, "vdim": diff_vdim, "scale": diff_dim ** -0.5,
+        "softcap": 30.0, "diff": 0.3,
+        "rot": {"base": 1000000.0, "dims": diff_dim, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+    mlps = [{"kind": "dense", "ff": dense_ff},
+            {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}]
+    kinds = [diff if i % 3 == 2 else latent(i - 1 if i % 3 == 1 else None) for i in range(layers)]
+    return {"architecture": "Rutevik", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "layers": [dict(kinds[i], mlp=mlps[i % 2]) for i in range(layers)]}
+
+
+# Rutevik at sizes that resemble a real model's layers, beside the Qwen3 shape of the same width and, with
+# --design-beside disunex, beside the design whose layers are closest (latent attention over one key head, routed
+# experts, a dense feed-forward of two matrices): the latent layers have Disunex's sizes without its window, the
+# differential attention has two maps of 64 a head on values of 128, which is one key row of 128 a kv head
+RUTEVIK_SHAPES = {
+    "2k": ("1.7b", dict(width=2048, heads=16, dim=64, rot=32, vdim=64, rank=96, q_rank=768, diff_heads=16, diff_kv_heads=4,
+                        diff_dim=64, diff_vdim=128, dense_ff=9216, experts=16, top=2, expert_ff=1024)),
+    "4k": ("8b", dict(width=4096, heads=32, dim=128, rot=64, vdim=128, rank=192, q_rank=1536, diff_heads=32, diff_kv_heads=8,
+                      diff_dim=64, diff_vdim=128, dense_ff=18432, experts=32, top=4, expert_ff=1536)),
+}
+
 DESIGNS = {"disunex": ("Disunex", DISUNEX_SHAPES, disunex_shape), "netovik": ("Netovik", NETOVIK_SHAPES, netovik_shape),
-           "sipilorn": ("Sipilorn", SIPILORN_SHAPES, sipilorn_shape)}
+           "sipilorn": ("Sipilorn", SIPILORN_SHAPES, sipilorn_shape), "rutevik": ("Rutevik", RUTEVIK_SHAPES, rutevik_shape)}
 
 
 def design_points(args):

@@ -108,14 +108,15 @@ def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
 # and 1.3e-2; a run prints what it saw at its end).
 # The nv configurations are sharpened more and norm every sublayer's output, per head in the recurrence, where
 # few terms can nearly cancel: float32 1.1e-5 at worst, bfloat16 3.7e-2 and 5.2e-2 at one request's second token.
+# The rv configurations: float32 5.1e-7 / 6.8e-7 / 7.2e-7 / 3.4e-6 for A / B / C / D, bfloat16 8.2e-3 / 7.8e-3 / 7.8e-3 / 2.6e-2.
 # float32: the engine differs from a float64 run by rounding only.  bfloat16: weights are the
 # same bfloat16 values in both runs; the engine rounds activations to bfloat16 between kernels
 # (relative step 2^-8).  One wrong page among a request's five moves the logits of these models
 # by 7e-2 and more.
 _TOL = {
-    "float32": {"rvA": 2e-5, "rvB": 2e-5, "rvC": 2e-5, "rvD": 2e-5, "spA": 8e-5, "spB": 3e-5, "spC": 3e-5, "spD": 3e-5, "spE": 3e-5, "nvA": 3e-5, "nvB": 3e-5, "nvC": 3e-5, "nvD": 3e-5, "dxP": 2.5e-6, "dxQ": 2.5e-6, "dxR": 2.5e-6, "dxS": 2.5e-6, "dxT": 2.5e-6, "A": 1e-6, "B": 2.5e-6, "C": 3e-6, "D": 2e-6, "B0": 2.5e-6, "E": 3e-6, "W": 7e-6, "mid": 1.2e-5,
+    "float32": {"rvA": 2e-6, "rvB": 2e-6, "rvC": 2e-6, "rvD": 8e-6, "spA": 8e-5, "spB": 3e-5, "spC": 3e-5, "spD": 3e-5, "spE": 3e-5, "nvA": 3e-5, "nvB": 3e-5, "nvC": 3e-5, "nvD": 3e-5, "dxP": 2.5e-6, "dxQ": 2.5e-6, "dxR": 2.5e-6, "dxS": 2.5e-6, "dxT": 2.5e-6, "A": 1e-6, "B": 2.5e-6, "C": 3e-6, "D": 2e-6, "B0": 2.5e-6, "E": 3e-6, "W": 7e-6, "mid": 1.2e-5,
                 "large": 1.2e-5},
-    "bfloat16": {"rvA": 5e-2, "rvB": 5e-2, "rvC": 5e-2, "rvD": 5e-2, "spA": 6e-2, "spB": 6e-2, "spC": 6e-2, "spD": 6e-2, "spE": 6e-2, "nvA": 7e-2, "nvB": 7e-2, "nvC": 7e-2, "nvD": 7e-2, "dxP": 2.5e-2, "dxQ": 2.5e-2, "dxR": 2.5e-2, "dxS": 2.5e-2, "dxT": 2.5e-2, "A": 1e-2, "B": 2e-2, "C": 1.8e-2, "D": 1.6e-2, "B0": 2e-2, "E": 1.5e-2, "W": 2.6e-2, "mid": 2.6e-2,
+    "bfloat16": {"rvA": 2e-2, "rvB": 2e-2, "rvC": 2e-2, "rvD": 5e-2, "spA": 6e-2, "spB": 6e-2, "spC": 6e-2, "spD": 6e-2, "spE": 6e-2, "nvA": 7e-2, "nvB": 7e-2, "nvC": 7e-2, "nvD": 7e-2, "dxP": 2.5e-2, "dxQ": 2.5e-2, "dxR": 2.5e-2, "dxS": 2.5e-2, "dxT": 2.5e-2, "A": 1e-2, "B": 2e-2, "C": 1.8e-2, "D": 1.6e-2, "B0": 2e-2, "E": 1.5e-2, "W": 2.6e-2, "mid": 2.6e-2,
                  "large": 2e-2},
 }
 

@@ -206,8 +206,7 @@ def test_the_test_configurations_differ_from_each_other():
 def test_the_sharpened_weights_show_a_lost_cache_a_wrong_map_and_a_wrong_source(tmp_path, name):
     """What the comparisons on the GPU rest on: in the plain implementation itself, a request that goes on without its
     earlier tokens, a reader that takes its own layer's input for the borrowed cache's, and a second map that is
-    left out each move some row of logits by more than four times (the map: twice) what any row may differ by in
-    bfloat16."""
+    left out each move some row of logits by more than four times what any row may differ by in bfloat16."""
     from helpers import rel_err, tol
     from rutevik_models import clear_tokens
     cfg, seed = RUTEVIK_CONFIGS[name]
@@ -237,4 +236,4 @@ def test_the_sharpened_weights_show_a_lost_cache_a_wrong_map_and_a_wrong_source(
     flat = copy.deepcopy(c)
     flat["layers"][j]["mixer"]["diff"] = 0.0            # lambda = e^-big - e^-big + 0 = 0
     out = plain.forward(flat, P2, toks)
-    assert max(rel_err(out[t], ref[t]) for t in range(len(toks))) > limit / 2
+    assert max(rel_err(out[t], ref[t]) for t in range(len(toks))) > limit
