@@ -44,42 +44,51 @@ __device__ __forceinline__ float diff_rotated(const float* __restrict__ x, const
     return first ? fmaf(v, c, -(o * s)) : fmaf(v, c, o * s);
 }
 
+// Blocks (token, y): y < q_blocks works through DQ_HEADS query heads (head 2 h + m holds map m at elements
+// m D .. m D + D - 1 and zeros elsewhere); the others are one kv head each: its key row and its value row into the
+// token's slot.  A thread's elements lie DQ_THREADS apart, so no index is divided.
+#define DQ_THREADS 128
+#define DQ_HEADS 8
+
 template <typename TC>
-__global__ __launch_bounds__(256) void diff_qkv_store_kernel(
+__global__ __launch_bounds__(DQ_THREADS) void diff_qkv_store_kernel(
     const float* __restrict__ proj, size_t row, const float* __restrict__ qb, const float* __restrict__ kb,
     const float* __restrict__ vb, const float* __restrict__ cos_sin, int rot_dims, int pairing, int max_pos,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, TC* __restrict__ q_out,
-    TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size, int H, int G, int D, int E, int P) {
-    const int t = blockIdx.x, tid = threadIdx.x;
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size, int H, int G, int D, int E, int P, int q_blocks) {
+    const int t = blockIdx.x, y = blockIdx.y, tid = threadIdx.x;
     const float* x = proj + (size_t)t * row;
     const int pos = min(max(positions[t], 0), max(max_pos - 1, 0));
     const DiffRot rot{(cos_sin && rot_dims) ? cos_sin + (size_t)pos * rot_dims : nullptr, rot_dims, pairing};
-    // queries: head 2 h + m holds map m at elements m D .. m D + D - 1 and zeros elsewhere
-    TC* qo = q_out + (size_t)t * 2 * H * P;
-    for (int i = tid; i < 2 * H * P; i += blockDim.x) {
-        const int hm = i / P, e2 = i - hm * P, m = hm & 1;
-        float v = 0.f;
-        if (e2 >= m * D && e2 < (m + 1) * D) v = diff_rotated(x + (size_t)hm * D, qb ? qb + (size_t)hm * D : nullptr, e2 - m * D, rot);
-        qo[i] = from_f32<TC>(v);
+    if (y < q_blocks) {
+        TC* qo = q_out + (size_t)t * 2 * H * P;
+        for (int hm = y * DQ_HEADS; hm < min(2 * H, (y + 1) * DQ_HEADS); ++hm) {
+            const int lo = (hm & 1) * D;
+            for (int e2 = tid; e2 < P; e2 += DQ_THREADS) {
+                float v = 0.f;
+                if (e2 >= lo && e2 < lo + D) v = diff_rotated(x + (size_t)hm * D, qb ? qb + (size_t)hm * D : nullptr, e2 - lo, rot);
+                qo[(size_t)hm * P + e2] = from_f32<TC>(v);
+            }
+        }
+        return;
     }
     const int slot = slots[t];
     if (slot < 0) return;      // (the whole block: a token that writes no key)
+    const int g = y - q_blocks;
     const int page = slot / page_size, off = slot - page * page_size;
-    const float* xk = x + (size_t)2 * H * D;
-    const float* xv = xk + (size_t)2 * G * D;
-    for (int i = tid; i < G * P; i += blockDim.x) {
-        const int g = i / P, e2 = i - g * P;
-        float v = 0.f;
+    const float* xk = x + (size_t)2 * H * D + (size_t)2 * g * D;
+    const float* xv = x + (size_t)2 * H * D + (size_t)2 * G * D + (size_t)g * E;
+    TC* kd = k_cache + (((size_t)page * G + g) * page_size + off) * P;
+    TC* vd = v_cache + ((size_t)page * G + g) * P * page_size + off;
+    for (int e2 = tid; e2 < P; e2 += DQ_THREADS) {
+        float k = 0.f;
         if (e2 < 2 * D) {
-            const int m = e2 / D;
-            v = diff_rotated(xk + (size_t)(2 * g + m) * D, kb ? kb + (size_t)(2 * g + m) * D : nullptr, e2 - m * D, rot);
+            const int m = e2 >= D ? 1 : 0;
+            k = diff_rotated(xk + (size_t)m * D, kb ? kb + (size_t)(2 * g + m) * D : nullptr, e2 - m * D, rot);
         }
-        k_cache[(((size_t)page * G + g) * page_size + off) * P + e2] = from_f32<TC>(v);
-    }
-    for (int i = tid; i < G * P; i += blockDim.x) {
-        const int g = i / P, e = i - g * P;
-        const float v = e < E ? xv[(size_t)g * E + e] + (vb ? vb[(size_t)g * E + e] : 0.f) : 0.f;
-        v_cache[(((size_t)page * G + g) * P + e) * page_size + off] = from_f32<TC>(v);
+        kd[e2] = from_f32<TC>(k);
+        const float v = e2 < E ? xv[e2] + (vb ? vb[(size_t)g * E + e2] : 0.f) : 0.f;
+        vd[(size_t)e2 * page_size] = from_f32<TC>(v);
     }
 }
 
@@ -96,12 +105,17 @@ TFF_API int tff_diff_qkv_store(const float* proj, size_t row, const float* qb, c
     TFF_REQUIRE(page_size > 0 && num_pages > 0, "diff_qkv_store: bad cache geometry");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    const int q_blocks = (2 * H + DQ_HEADS - 1) / DQ_HEADS;
+    TFF_REQUIRE(q_blocks + G <= 65535, "diff_qkv_store: too many heads");
+    const dim3 grid(T, q_blocks + G);
     if (dtype == TFF_F32)
-        diff_qkv_store_kernel<float><<<T, 256, 0, s>>>(proj, row, qb, kb, vb, cos_sin, rot_dims, pairing, max_pos, positions, slots,
-                                                       (float*)q_out, (float*)k_cache, (float*)v_cache, page_size, H, G, D, E, P);
+        diff_qkv_store_kernel<float><<<grid, DQ_THREADS, 0, s>>>(proj, row, qb, kb, vb, cos_sin, rot_dims, pairing, max_pos, positions,
+                                                                 slots, (float*)q_out, (float*)k_cache, (float*)v_cache, page_size,
+                                                                 H, G, D, E, P, q_blocks);
     else if (dtype == TFF_BF16)
-        diff_qkv_store_kernel<bf16_t><<<T, 256, 0, s>>>(proj, row, qb, kb, vb, cos_sin, rot_dims, pairing, max_pos, positions, slots,
-                                                        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, H, G, D, E, P);
+        diff_qkv_store_kernel<bf16_t><<<grid, DQ_THREADS, 0, s>>>(proj, row, qb, kb, vb, cos_sin, rot_dims, pairing, max_pos, positions,
+                                                                  slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                                                  page_size, H, G, D, E, P, q_blocks);
     else
         return tff_fail("diff_qkv_store: unknown dtype %d", dtype);
     return tff_check_launch("diff_qkv_store");
