@@ -116,14 +116,14 @@ def rutevik_shape(width, heads, dim, rot, vdim, rank, q_rank, diff_heads, diff_k
     then a differential attention, and so on; dense feed-forwards and mixtures of experts in turn."""
     def latent(source):
         m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "q_rank": q_rank,
-             "scale": (dim + rot) ** -0.5, "rot": {"base": 20000.0, "dims": rot}}
+             "scale": (dim + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}
         if source is not None:
             m["kv_from"] = source
         return {"type": "latent_attention", "mixer": m}
     diff = {"type": "attention", "mixer": {
         "heads": diff_heads, "kv_heads": diff_kv_heads, "dim": diff_dim, "vdim": diff_vdim, "scale": diff_dim ** -0.5,
-        "softcap": 30.0, "diff": 0.3,
-        "rot": {"base": 1000000.0, "dims": diff_dim, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+        "softcap": 50.0, "diff": 0.25,
+        "rot": {"base": 500000.0, "dims": diff_dim, "scaling": {"factor": 4.0, "low": 1.0, "high": 2.0, "original": 8192}}}}
     mlps = [{"kind": "dense", "ff": dense_ff},
             {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}]
     kinds = [diff if i % 3 == 2 else latent(i - 1 if i % 3 == 1 else None) for i in range(layers)]
