@@ -195,7 +195,8 @@ def _latent_part(W, H, D, R, E, rank, q_rank, scale, base, eps, dtype, seed, sha
     (3, 16, 8, 24, 40, 24, 16),
     (1, 64, 32, 64, 64, 16, 8),
     (5, 12, 6, 20, 30, 18, 32),          # no size a multiple of 8
-    (8, 64, 32, 64, 160, 96, 16)])       # a key of 192
+    (8, 64, 32, 64, 160, 96, 16),        # a key of 192
+    (2, 32, 64, 40, 272, 48, 16)])       # a key of 336, beyond the sizes of the matrix-core attention
 def test_latent_attention_with_a_latent_query_and_a_reader(H, D, R, E, rank, q_rank, page, dtype, limit):
     """Queries through a normed latent vector, keys and values through another, the rotated part turned in halves;
     a second attention with its own queries and up-projections reads the cache the first one fills.  A prompt in
@@ -242,7 +243,9 @@ def _diff_part(W, H, G, D, E, scale, diff, rot, softcap, scaling, eps, dtype, se
     (2, 1, 32, 48, (32, 1e6), None, None, 8),                    # values narrower than two maps, no cap
     (6, 6, 8, 8, (8, 50.0), 2.0, None, 32),                      # heads that are not grouped, a tight cap
     (3, 1, 12, 20, (4, 1e4), 12.0, (2.0, 1.0, 3.0, 16), 16),     # no multiples of 8
-    (8, 2, 64, 128, (64, 1e4), 20.0, (8.0, 1.0, 4.0, 64), 16)])  # the sizes of a real model
+    (8, 2, 64, 128, (64, 1e4), 20.0, (8.0, 1.0, 4.0, 64), 16),   # the sizes of a real model
+    (2, 1, 128, 96, (32, 1e4), 9.0, None, 16),                   # a key row of 256: capped scores on the general kernel
+    (2, 2, 24, 200, (24, 1e3), None, None, 8)])                  # values far wider than two maps
 def test_differential_attention_part(H, G, D, E, rot, softcap, scaling, page, dtype, limit):
     """Two score maps a head with biases, rotation, a cap on the scores, the difference with lambda, the norm over
     the head, the gate: a prompt in one step, as portions down to two tokens, and as a portion followed by single
