@@ -75,6 +75,29 @@ def test_norm_without_statistics(W):
     assert torch.equal(o_many[:n], o_few) and torch.equal(r_many[:n], r_few)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (8, 4096, 1024), (16, 320, 72), (5, 2048, 4096)])
+def test_norm_in_the_epilogue_of_a_product_of_few_rows(M, N, K):
+    """A product of up to 16 bfloat16 rows that has not run yet runs with the sum into the stream and the norm in
+    its epilogue: the same stream and the same rows as the product followed by the norm's own kernel."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(M * N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    wm = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    pw = ops.pack_weight(wm.to(DEV))
+    resid0 = torch.randn(M, N, generator=g) * 2
+    w, b, alpha = (1 + 0.3 * torch.randn(N, generator=g)).to(DEV), torch.randn(N, generator=g).to(DEV), 0.41
+    pending = ops.linear(x, pw, out_dtype=torch.float32, partials=True)
+    plain_run = ops.linear(x, pw, out_dtype=torch.float32)
+    r1, r2 = resid0.clone().to(DEV), resid0.clone().to(DEV)
+    fused = ops.add_dyt(r1, pending, alpha, w, b, torch.bfloat16)
+    apart = ops.add_dyt(r2, plain_run, alpha, w, b, torch.bfloat16)
+    if isinstance(pending, ops.PendingProduct):
+        assert torch.equal(r1, r2) and torch.equal(fused, apart)
+    total = resid0.double() + x.double().cpu() @ wm.double().T
+    assert _err(r1, total) < 2e-6
+    assert _err(fused.float(), plain.dyt(total, alpha, w.double().cpu(), b.double().cpu())) < 5e-3
+
+
 def test_square_of_relu():
     ops = _ops()
     z = torch.linspace(-6, 6, 2001)

@@ -734,6 +734,9 @@ static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, i
 //      multiplies its float32 accumulators by the row's factor before anything else is done
 //      to them.
 // The sum of squares is over the float32 residual stream, as in the norm's own kernel.
+//   3, the product before a norm that has no statistics (tanh(alpha v) w + b element by element): its
+//      epilogue adds its result to the residual stream in place and writes the norm of the sum as the
+//      bfloat16 input of the next product, whole: there is no factor to leave to anyone.
 struct SkinnyFuse {
     const float* ss_in;     // EPI 1: [16][ss_stride] sums of squares, ss_count of them a row
     int ss_stride, ss_count;
@@ -743,6 +746,8 @@ struct SkinnyFuse {
     bf16_t* x_out;          // [M, N]
     float* ss_out;          // [16][ss_out_stride]
     int ss_out_stride;
+    const float* bias;      // EPI 3: [N], and the scalar inside the tanh
+    float alpha;
 };
 
 template <int MT, int R, int UNROLL, int KSPLIT, int NSETS, bool GLU, typename TC, bool RING = false, int EPI = 0>
@@ -750,7 +755,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out, SkinnyFuse fz) {
     static_assert(EPI == 0 || MT == 1, "the fused norm is for up to 16 rows");
-    static_assert(EPI != 2 || !GLU, "the product before a norm has a plain float32 result");
+    static_assert(EPI < 2 || !GLU, "the product before a norm has a plain float32 result");
     constexpr int SK_WAVES = KSPLIT * NSETS;
     static_assert(!GLU || (R == 1 && NSETS % 2 == 0), "a gate and its up group are one row group each");
     __shared__ floatx4 part[SK_WAVES][R * MT][64];
@@ -783,9 +788,11 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     // What the epilogue needs from memory is asked for first, so that it has arrived long
     // before the stream of W ends.
     float row_scale = 1.f;
-    float4 resid_in[R], normw_in[R];
+    float4 resid_in[R], normw_in[R], bias_in[EPI == 3 ? R : 1];
 #pragma unroll
     for (int r = 0; r < R; ++r) resid_in[r] = normw_in[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int r = 0; r < (EPI == 3 ? R : 1); ++r) bias_in[r] = make_float4(0.f, 0.f, 0.f, 0.f);
     // EPI 1: lane (fr, fg) of a set's first wave adds every fourth group of four sums of row fr,
     // then the four lanes of a row meet: the same order in every block.  The loads are issued
     // here, ahead of the stream of W, and added up (TFF_ROW_SCALE) when that stream has ended.
@@ -823,7 +830,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
             row_scale = rsqrtf(ssum * fz.inv_dim + fz.eps);                                        \
         }                                                                                          \
     }
-    if constexpr (EPI == 2) {
+    if constexpr (EPI >= 2) {
         if (wave == 0) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -831,6 +838,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
                 if (fr < M && n < N) {
                     resid_in[r] = *reinterpret_cast<const float4*>(fz.resid + (size_t)fr * N + n);
                     normw_in[r] = *reinterpret_cast<const float4*>(fz.norm_w + n);
+                    if constexpr (EPI == 3) bias_in[r] = *reinterpret_cast<const float4*>(fz.bias + n);
                 }
             }
         }
@@ -975,6 +983,18 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
                         ss += __shfl_xor(ss, 16, 64);
                         ss += __shfl_xor(ss, 32, 64);
                         if (fg == 0 && nb0 + r < NB) fz.ss_out[(size_t)fr * fz.ss_out_stride + nb0 + r] = ss;
+                    } else if constexpr (EPI == 3) {
+                        if (m < M && n < N) {
+                            const float4 sum = make_float4(resid_in[r].x + v[0], resid_in[r].y + v[1],
+                                                           resid_in[r].z + v[2], resid_in[r].w + v[3]);
+                            *reinterpret_cast<float4*>(fz.resid + (size_t)m * N + n) = sum;
+                            union { bf16_t h[4]; uint2 u; } pk;
+                            pk.h[0] = (bf16_t)fmaf(tanhf(fz.alpha * sum.x), normw_in[r].x, bias_in[r].x);
+                            pk.h[1] = (bf16_t)fmaf(tanhf(fz.alpha * sum.y), normw_in[r].y, bias_in[r].y);
+                            pk.h[2] = (bf16_t)fmaf(tanhf(fz.alpha * sum.z), normw_in[r].z, bias_in[r].z);
+                            pk.h[3] = (bf16_t)fmaf(tanhf(fz.alpha * sum.w), normw_in[r].w, bias_in[r].w);
+                            *reinterpret_cast<uint2*>(fz.x_out + (size_t)m * N + n) = pk.u;
+                        }
                     } else if (m < M && n < N) {
                         store4<TC>(C + (size_t)m * N + n, v, n, N, vec);
                     }
@@ -989,11 +1009,11 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
     const int NB = (N + 15) / 16, KB = (K + 31) / 32;
     const int per_block = NSETS * R;
     const dim3 grid((NB + per_block - 1) / per_block);
-    const SkinnyFuse fz = fuse ? *fuse : SkinnyFuse{nullptr, 0, 0, 0.f, 0.f, nullptr, nullptr, nullptr, nullptr, 0};
+    const SkinnyFuse fz = fuse ? *fuse : SkinnyFuse{nullptr, 0, 0, 0.f, 0.f, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f};
     if (c_dtype == TFF_F32)
         gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, float, RING, EPI>
             <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, fz);
-    else if constexpr (EPI != 2)
+    else if constexpr (EPI < 2)
         gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, bf16_t, RING, EPI>
             <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, fz);
     else
@@ -1184,7 +1204,7 @@ template <int EPI>
 static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
                       int glu_out, hipStream_t s, const SkinnyFuse* fuse) {
     if (glu_out > 0) {
-        if constexpr (EPI != 2) {
+        if constexpr (EPI < 2) {
             if (N >= 8 * 1024)
                 return launch_skinny<1, 1, 8, 1, 2, true, true, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
             // A wave takes a quarter of K in groups of k-steps whose loads are issued together, and
@@ -1332,8 +1352,22 @@ TFF_API int tff_gemm_residual_prenorm(const void* A, const void* Wp, int M, int 
                 "ss_out needs %d floats a row, has %d", N, (N + 15) / 16, ss_stride);
     TFF_REQUIRE(((uintptr_t)resid % 16) == 0 && ((uintptr_t)norm_w % 16) == 0 && ((uintptr_t)x_out % 8) == 0,
                 "gemm_residual_prenorm: operands must be 16-byte aligned");
-    SkinnyFuse fz{nullptr, 0, 0, 0.f, 0.f, resid, norm_w, (bf16_t*)x_out, ss_out, ss_stride};
+    SkinnyFuse fz{nullptr, 0, 0, 0.f, 0.f, resid, norm_w, (bf16_t*)x_out, ss_out, ss_stride, nullptr, 0.f};
     return skinny_for<2>((const bf16_t*)A, (const bf16_t*)Wp, resid, M, N, K, lda, TFF_F32, 0, (hipStream_t)stream, &fz);
+}
+
+// resid[M, N] += A . W^T (bfloat16 A and packed W, float32 sums); x_out[M, N] = bfloat16 of
+// tanh(alpha * resid) * norm_w + bias over the new resid: the norm without statistics in the epilogue of the
+// product before it.  Up to 16 rows; N a multiple of 8.
+TFF_API int tff_gemm_residual_dyt(const void* A, const void* Wp, int M, int N, int K, int lda, float* resid, float alpha,
+                                  const float* norm_w, const float* bias, void* x_out, tff_stream_t stream) {
+    if (int rc = check_fused_operands("gemm_residual_dyt", A, Wp, M, N, K, lda)) return rc;
+    TFF_REQUIRE(resid && norm_w && bias && x_out, "gemm_residual_dyt: null pointer");
+    TFF_REQUIRE(N % 8 == 0, "gemm_residual_dyt: N=%d must be a multiple of 8", N);
+    TFF_REQUIRE(((uintptr_t)resid % 16) == 0 && ((uintptr_t)norm_w % 16) == 0 && ((uintptr_t)bias % 16) == 0 &&
+                ((uintptr_t)x_out % 8) == 0, "gemm_residual_dyt: operands must be 16-byte aligned");
+    SkinnyFuse fz{nullptr, 0, 0, 0.f, 0.f, resid, norm_w, (bf16_t*)x_out, nullptr, 0, bias, alpha};
+    return skinny_for<3>((const bf16_t*)A, (const bf16_t*)Wp, resid, M, N, K, lda, TFF_F32, 0, (hipStream_t)stream, &fz);
 }
 
 // C = rstd[m] * (A . W^T) with rstd[m] = rsqrt(sum_g ss[m][g] / dim + eps), g < ss_count: the product
@@ -1360,7 +1394,7 @@ TFF_API int tff_gemm_row_scaled(const void* A, const void* Wp, void* C, int M, i
             return launch_w4<2, 5, true, 1, true, 2>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
         return launch_w4<4, 5, true, 1, true, 2>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
     }
-    SkinnyFuse fz{ss, ss_stride, ss_count, 1.0f / (float)dim, eps, nullptr, nullptr, nullptr, nullptr, 0};
+    SkinnyFuse fz{ss, ss_stride, ss_count, 1.0f / (float)dim, eps, nullptr, nullptr, nullptr, nullptr, 0, nullptr, 0.f};
     return skinny_for<1>((const bf16_t*)A, (const bf16_t*)Wp, C, M, N, K, lda, c_dtype, glu_out, (hipStream_t)stream, &fz);
 }
 

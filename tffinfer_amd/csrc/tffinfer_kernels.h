@@ -56,6 +56,11 @@ TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int g
 TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int keep_partials, int* tile_rows, int* tile_cols,
                           int* splits);
 
+// resid[M, N] += A . W^T; x_out[M, N] = bfloat16 of tanh(alpha * resid) * norm_w + bias over the new resid: a norm
+// without statistics in the epilogue of the product before it.  Up to 16 rows, bfloat16, N a multiple of 8.
+TFF_API int tff_gemm_residual_dyt(const void* A, const void* Wp, int M, int N, int K, int lda, float* resid, float alpha,
+                                  const float* norm_w, const float* bias, void* x_out, tff_stream_t stream);
+
 // An RMS norm between two bfloat16 products of up to 16 rows, taken into them (its per-row
 // factor commutes with the product after it):
 //   tff_gemm_residual_prenorm: resid[M, N] += A . W^T in place (float32); x_out[M, N] = bfloat16

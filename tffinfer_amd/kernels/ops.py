@@ -1595,6 +1595,16 @@ def add_dyt(resid: torch.Tensor, delta, alpha: float, weight: torch.Tensor, bias
         _req(w, f"add_dyt {nm}", torch.float32, 1)
         if w.numel() != H:
             raise _lib.KernelError(f"add_dyt: {nm} has {w.numel()} elements, rows have {H}")
+    if isinstance(delta, PendingProduct) and rows is None and out_dtype == torch.bfloat16 \
+            and tuple(delta.shape) == tuple(resid.shape):
+        # a product of a few rows that has not run: it runs with the sum and the norm in its epilogue
+        p = delta
+        M, K = p.x.shape
+        out = torch.empty(M, H, dtype=torch.bfloat16, device=resid.device)
+        _lib.check(_lib.load().tff_gemm_residual_dyt(p.x.data_ptr(), p.weight.data_ptr(), M, H, K,
+                                                     p.x.stride(0) if M > 1 else K, resid.data_ptr(), float(alpha),
+                                                     weight.data_ptr(), bias.data_ptr(), out.data_ptr(), _stream()))
+        return out
     terms = delta.terms if isinstance(delta, PendingTerms) else ([] if delta is None else [delta])
     d = [_planes_of(t, resid.shape, "add_dyt term") for t in terms] + [(None, 0, 0)] * 2
     if rows is not None:
