@@ -219,7 +219,8 @@ def _latent_part(W, H, D, R, E, rank, q_rank, scale, base, eps, dtype, seed, sha
     (1, 64, 32, 64, 64, 16, 8),
     (5, 12, 6, 20, 30, 18, 32),          # no size a multiple of 8
     (8, 64, 32, 64, 160, 96, 16),        # a key of 192
-    (2, 32, 64, 40, 272, 48, 16)])       # a key of 336, beyond the sizes of the matrix-core attention
+    (2, 32, 64, 40, 272, 48, 16),        # a key of 336, beyond the sizes of the matrix-core attention
+    (2, 16, 64, 24, 512, 32, 16)])       # a key of 576
 def test_latent_attention_with_a_latent_query_and_a_reader(H, D, R, E, rank, q_rank, page, dtype, limit):
     """Queries through a normed latent vector, keys and values through another, the rotated part turned in halves;
     a second attention with its own queries and up-projections reads the cache the first one fills.  A prompt in

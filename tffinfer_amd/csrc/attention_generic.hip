@@ -15,15 +15,15 @@
 #include "common.h"
 #include "tffinfer_kernels.h"
 
-#define AG_MAX_D 512
+#define AG_MAX_D 1024     // (a kernel for head sizes up to 512, one for those beyond: the accumulators are registers)
 
-template <typename T, typename TC>
+template <typename T, typename TC, int MAXD>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, const TC* __restrict__ k_cache,
     const TC* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
     const int32_t* __restrict__ token_req, const int32_t* __restrict__ positions, int nq, int nkv,
     int d, int page_size, int window, float scale, const float* __restrict__ sinks, float softcap) {
-    __shared__ float qs[AG_MAX_D];
+    __shared__ float qs[MAXD];
     __shared__ long long voff[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int G = nq / nkv;
@@ -38,9 +38,9 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     __syncthreads();
 
     float m = -INFINITY, l = 0.f;
-    float acc[AG_MAX_D / 64];
+    float acc[MAXD / 64];
 #pragma unroll
-    for (int i = 0; i < AG_MAX_D / 64; ++i) acc[i] = 0.f;
+    for (int i = 0; i < MAXD / 64; ++i) acc[i] = 0.f;
 
     for (int base = lo; base <= pos; base += 64) {
         const int j = base + lane;
@@ -68,12 +68,12 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         __syncthreads();
         const int nvalid = min(64, pos - base + 1);
 #pragma unroll
-        for (int i = 0; i < AG_MAX_D / 64; ++i) acc[i] *= corr;
+        for (int i = 0; i < MAXD / 64; ++i) acc[i] *= corr;
         for (int jj = 0; jj < nvalid; ++jj) {
             const float pj = __shfl(p, jj, 64);
             const TC* vp = v_cache + voff[jj];
 #pragma unroll
-            for (int i = 0; i < AG_MAX_D / 64; ++i) {
+            for (int i = 0; i < MAXD / 64; ++i) {
                 const int e = lane + 64 * i;
                 if (e < d) acc[i] = fmaf(pj, to_f32(vp[(long long)e * page_size]), acc[i]);
             }
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     if (sinks) l += expf(sinks[h] - m);
     const float inv = 1.0f / l;
 #pragma unroll
-    for (int i = 0; i < AG_MAX_D / 64; ++i) {
+    for (int i = 0; i < MAXD / 64; ++i) {
         const int e = lane + 64 * i;
         if (e < d) op[e] = from_f32<T>(acc[i] * inv);
     }
@@ -111,16 +111,17 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out, const 
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(T, nq);
-    if (dtype == TFF_F32)
-        attention_generic_kernel<float, float><<<grid, 64, 0, s>>>(
-            (const float*)q, q_stride, (float*)out, (const float*)k_cache, (const float*)v_cache,
-            block_tables, bt_stride, token_req, positions, nq, nkv, d, page_size, window, scale, sinks, softcap);
-    else if (dtype == TFF_BF16)
-        attention_generic_kernel<bf16_t, bf16_t><<<grid, 64, 0, s>>>(
-            (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache,
-            (const bf16_t*)v_cache, block_tables, bt_stride, token_req, positions, nq, nkv, d,
-            page_size, window, scale, sinks, softcap);
-    else
+#define TFF_AG(TT, MAXD)                                                                                            \
+    attention_generic_kernel<TT, TT, MAXD><<<grid, 64, 0, s>>>((const TT*)q, q_stride, (TT*)out, (const TT*)k_cache, \
+                                                              (const TT*)v_cache, block_tables, bt_stride, token_req, \
+                                                              positions, nq, nkv, d, page_size, window, scale, sinks, softcap)
+    if (dtype == TFF_F32) {
+        if (d <= 512) TFF_AG(float, 512); else TFF_AG(float, AG_MAX_D);
+    } else if (dtype == TFF_BF16) {
+        if (d <= 512) TFF_AG(bf16_t, 512); else TFF_AG(bf16_t, AG_MAX_D);
+    } else {
         return tff_fail("attention: unknown dtype %d", dtype);
+    }
+#undef TFF_AG
     return tff_check_launch("attention_generic");
 }
